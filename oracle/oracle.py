@@ -1,0 +1,340 @@
+"""CPU checker for the transformer-block hot path -- TEST INFRASTRUCTURE ONLY.
+
+Two things live here:
+
+* ``C`` -- ctypes bindings for ``libdtoracle.so`` (built from ``dt_oracle.c``,
+  the C restatement whose header lists what each function follows in the
+  reference and what pins it).
+* ``np_*`` -- a second, independently written numpy restatement of the
+  integer parts (index packing, palette lookup) and float64 versions of the
+  floating-point parts.  The tests pin the C code against these, against
+  hand-built byte vectors and against closed forms, so that a slip in either
+  one (wrong bit order, wrong block stride, transposed operand) shows up.
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module.  The product path never does.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "libdtoracle.so")
+
+_u8p = ctypes.POINTER(ctypes.c_uint8)
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+_f32p = ctypes.POINTER(ctypes.c_float)
+_i32p = ctypes.POINTER(ctypes.c_int)
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+
+
+def build(force: bool = False) -> str:
+    """Compile libdtoracle.so with the Makefile next to this file."""
+    if force or not os.path.exists(_LIB) or os.path.getmtime(_LIB) < os.path.getmtime(
+        os.path.join(_HERE, "dt_oracle.c")
+    ):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libdtoracle.so"], stdout=subprocess.DEVNULL)
+    return _LIB
+
+
+def _ptr(a: np.ndarray, typ):
+    return a.ctypes.data_as(typ)
+
+
+class _C:
+    """Thin typed wrapper over the C oracle."""
+
+    def __init__(self):
+        self._lib = None
+
+    @property
+    def lib(self):
+        if self._lib is None:
+            if not os.path.exists(_LIB):
+                build()
+            lib = ctypes.CDLL(_LIB)
+            lib.dto_qx_bytes.restype = _i64
+            lib.dto_qx_bytes.argtypes = [_int, _int, _i64]
+            lib.dto_pack_indices.argtypes = [_int, _u8p, _i64, _u8p]
+            lib.dto_unpack_indices.argtypes = [_int, _u8p, _i64, _u8p]
+            lib.dto_palettize_pack.argtypes = [_int, _int, _i64, _u16p, _u8p, _u8p]
+            lib.dto_depalettize.argtypes = [_int, _int, _i64, _u8p, _u16p]
+            lib.dto_dense.argtypes = [_i64, _i64, _i64, _u16p, _i64, _u16p, _u16p, _u16p, _i64]
+            lib.dto_dense_qx.argtypes = [_i64, _i64, _i64, _u16p, _i64, _u8p, _int, _int, _u16p, _u16p, _i64]
+            lib.dto_rmsnorm.restype = None
+            lib.dto_rmsnorm.argtypes = [_i64, _i64, _u16p, _i64, _u16p, ctypes.c_float, _u16p, _i64]
+            lib.dto_cmul.restype = None
+            lib.dto_cmul.argtypes = [_i64, _i64, _i64, _u16p, _i64, _i64, _u16p, _i64, _u16p, _i64, _i64]
+            lib.dto_rope_flux.argtypes = [_int, _int, _int, _int, _i32p, _int, _f32p]
+            lib.dto_rope_wan.argtypes = [_int, _int, _int, _int, _f32p]
+            lib.dto_sdpa.argtypes = (
+                [_int, _int, _int, _int, _i64, _i64]
+                + [_u16p, _i64, _i64, _i64] * 4
+                + [ctypes.c_float, _int]
+            )
+            lib.dto_dense_instruction_count.restype = _i64
+            lib.dto_dense_instruction_count.argtypes = [_i64, _i64, _i64]
+            lib.dto_sdpa_instruction_count.restype = _i64
+            lib.dto_sdpa_instruction_count.argtypes = [_i64] * 5
+            lib.dto_h2f.restype = ctypes.c_float
+            lib.dto_h2f.argtypes = [ctypes.c_uint16]
+            lib.dto_f2h.restype = ctypes.c_uint16
+            lib.dto_f2h.argtypes = [ctypes.c_float]
+            self._lib = lib
+        return self._lib
+
+    # -- layout ---------------------------------------------------------
+    def qx_bytes(self, qbits, nib, count):
+        return int(self.lib.dto_qx_bytes(qbits, nib, count))
+
+    def pack_indices(self, qbits, idx):
+        idx = np.ascontiguousarray(idx, dtype=np.uint8)
+        out = np.zeros((idx.size * qbits + 7) // 8, dtype=np.uint8)
+        self.lib.dto_pack_indices(qbits, _ptr(idx, _u8p), idx.size, _ptr(out, _u8p))
+        return out
+
+    def unpack_indices(self, qbits, packed, n):
+        packed = np.ascontiguousarray(packed, dtype=np.uint8)
+        out = np.zeros(n, dtype=np.uint8)
+        self.lib.dto_unpack_indices(qbits, _ptr(packed, _u8p), n, _ptr(out, _u8p))
+        return out
+
+    def palettize_pack(self, qbits, nib, palettes, idx):
+        """palettes: float16 [nblocks, 2^q]; idx: uint8 [count] -> packed uint8 buffer."""
+        idx = np.ascontiguousarray(idx, dtype=np.uint8).reshape(-1)
+        count = idx.size
+        palettes = np.ascontiguousarray(palettes, dtype=np.float16)
+        nblocks = (count + nib - 1) // nib
+        assert palettes.shape == (nblocks, 1 << qbits), palettes.shape
+        out = np.zeros(self.qx_bytes(qbits, nib, count), dtype=np.uint8)
+        rc = self.lib.dto_palettize_pack(
+            qbits, nib, count, _ptr(palettes.view(np.uint16), _u16p), _ptr(idx, _u8p), _ptr(out, _u8p)
+        )
+        assert rc == 0
+        return out
+
+    def depalettize(self, qbits, nib, count, packed):
+        packed = np.ascontiguousarray(packed, dtype=np.uint8)
+        out = np.zeros(count, dtype=np.uint16)
+        rc = self.lib.dto_depalettize(qbits, nib, count, _ptr(packed, _u8p), _ptr(out, _u16p))
+        assert rc == 0
+        return out.view(np.float16)
+
+    # -- float ops ------------------------------------------------------
+    def dense(self, X, W, bias=None):
+        """X [M,K] f16 (rows may be strided), W [N,K] f16 -> Y [M,N] f16."""
+        assert X.dtype == np.float16 and W.dtype == np.float16
+        M, K = X.shape
+        N = W.shape[0]
+        assert W.shape == (N, K) and X.strides[1] == 2
+        W = np.ascontiguousarray(W)
+        Y = np.zeros((M, N), dtype=np.float16)
+        b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float16)
+        rc = self.lib.dto_dense(
+            M, N, K, _ptr(X.view(np.uint16), _u16p), X.strides[0] // 2 if M else K,
+            _ptr(W.view(np.uint16), _u16p), None if b is None else _ptr(b.view(np.uint16), _u16p),
+            _ptr(Y.view(np.uint16), _u16p), N,
+        )
+        assert rc == 0
+        return Y
+
+    def dense_qx(self, X, packed, qbits, nib, N, bias=None):
+        assert X.dtype == np.float16
+        X = np.ascontiguousarray(X)
+        M, K = X.shape
+        packed = np.ascontiguousarray(packed, dtype=np.uint8)
+        Y = np.zeros((M, N), dtype=np.float16)
+        b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float16)
+        rc = self.lib.dto_dense_qx(
+            M, N, K, _ptr(X.view(np.uint16), _u16p), K, _ptr(packed, _u8p), qbits, nib,
+            None if b is None else _ptr(b.view(np.uint16), _u16p), _ptr(Y.view(np.uint16), _u16p), N,
+        )
+        assert rc == 0
+        return Y
+
+    def rmsnorm(self, x, gamma, eps=1e-6):
+        """x [..., width] f16 contiguous; normalises the last axis."""
+        x = np.ascontiguousarray(x, dtype=np.float16)
+        width = x.shape[-1]
+        rows = x.size // width
+        y = np.zeros_like(x)
+        g = None if gamma is None else np.ascontiguousarray(gamma, dtype=np.float16)
+        self.lib.dto_rmsnorm(
+            rows, width, _ptr(x.view(np.uint16), _u16p), width,
+            None if g is None else _ptr(g.view(np.uint16), _u16p), eps, _ptr(y.view(np.uint16), _u16p), width,
+        )
+        return y
+
+    def cmul(self, x, rot):
+        """x [S,H,D] f16, rot [S,D] f16 -> [S,H,D]."""
+        x = np.ascontiguousarray(x, dtype=np.float16)
+        rot = np.ascontiguousarray(rot, dtype=np.float16)
+        S, H, D = x.shape
+        assert rot.shape == (S, D)
+        y = np.zeros_like(x)
+        self.lib.dto_cmul(
+            S, H, D, _ptr(x.view(np.uint16), _u16p), H * D, D, _ptr(rot.view(np.uint16), _u16p), D,
+            _ptr(y.view(np.uint16), _u16p), H * D, D,
+        )
+        return y
+
+    def rope_flux(self, height, width, token_length, channels=128, ref_sizes=()):
+        n = token_length + height * width + sum(h * w for h, w in ref_sizes)
+        out = np.zeros((n, channels), dtype=np.float32)
+        ref = np.asarray([v for hw in ref_sizes for v in hw], dtype=np.int32)
+        rc = self.lib.dto_rope_flux(
+            height, width, token_length, len(ref_sizes), _ptr(ref, _i32p) if len(ref) else None, channels,
+            _ptr(out, _f32p),
+        )
+        assert rc == 0
+        return out
+
+    def rope_wan(self, height, width, time, channels=128):
+        out = np.zeros((time * height * width, channels), dtype=np.float32)
+        rc = self.lib.dto_rope_wan(height, width, time, channels, _ptr(out, _f32p))
+        assert rc == 0
+        return out
+
+    def sdpa(self, q, k, v, scale, round_mid=0):
+        """q [B,Sq,Hq,D], k/v [B,Skv,Hk,D] f16 (any strides with D contiguous) -> [B,Sq,Hq,D]."""
+        for t in (q, k, v):
+            assert t.dtype == np.float16 and t.ndim == 4 and (t.shape[3] == 1 or t.strides[3] == 2)
+        B, Sq, Hq, D = q.shape
+        _, Skv, Hk, _ = k.shape
+        o = np.zeros((B, Sq, Hq, D), dtype=np.float16)
+
+        def st(t):
+            return [t.strides[0] // 2, t.strides[1] // 2, t.strides[2] // 2]
+
+        rc = self.lib.dto_sdpa(
+            B, Hq, Hk, D, Sq, Skv,
+            _ptr(q.view(np.uint16), _u16p), *st(q),
+            _ptr(k.view(np.uint16), _u16p), *st(k),
+            _ptr(v.view(np.uint16), _u16p), *st(v),
+            _ptr(o.view(np.uint16), _u16p), *st(o),
+            float(scale), int(round_mid),
+        )
+        assert rc == 0
+        return o
+
+    def dense_instruction_count(self, rows, inp, out):
+        return int(self.lib.dto_dense_instruction_count(rows, inp, out))
+
+    def sdpa_instruction_count(self, b, h, d, sa, sb):
+        return int(self.lib.dto_sdpa_instruction_count(b, h, d, sa, sb))
+
+
+C = _C()
+
+
+# ----------------------------------------------------------------------------
+# Independent numpy restatement (bit-level parts exact, float parts in float64)
+# ----------------------------------------------------------------------------
+
+def np_pack_indices(qbits: int, idx) -> np.ndarray:
+    """MSB-first bit stream built with numpy's own bit packer."""
+    idx = np.asarray(idx, dtype=np.uint8).reshape(-1)
+    bits = np.unpackbits(idx[:, None], axis=1, bitorder="big")[:, 8 - qbits:]
+    return np.packbits(bits.reshape(-1), bitorder="big")
+
+
+def np_unpack_indices(qbits: int, packed, n: int) -> np.ndarray:
+    bits = np.unpackbits(np.asarray(packed, dtype=np.uint8), bitorder="big")[: n * qbits]
+    weights = (1 << np.arange(qbits - 1, -1, -1)).astype(np.uint16)
+    return (bits.reshape(n, qbits).astype(np.uint16) * weights).sum(axis=1).astype(np.uint8)
+
+
+def np_palettize_pack(qbits: int, nib: int, palettes, idx) -> np.ndarray:
+    idx = np.asarray(idx, dtype=np.uint8).reshape(-1)
+    palettes = np.asarray(palettes, dtype=np.float16)
+    chunks = []
+    for b in range((idx.size + nib - 1) // nib):
+        chunks.append(palettes[b].view(np.uint8).reshape(-1))
+        chunks.append(np_pack_indices(qbits, idx[b * nib:(b + 1) * nib]))
+    return np.concatenate(chunks) if chunks else np.zeros(0, np.uint8)
+
+
+def np_depalettize(qbits: int, nib: int, count: int, packed) -> np.ndarray:
+    packed = np.asarray(packed, dtype=np.uint8)
+    out = np.zeros(count, dtype=np.float16)
+    pos = 0
+    palbytes = 2 << qbits
+    for b in range((count + nib - 1) // nib):
+        n = min(nib, count - b * nib)
+        pal = packed[pos:pos + palbytes].view(np.float16)
+        pos += palbytes
+        nbytes = (n * qbits + 7) // 8
+        out[b * nib:b * nib + n] = pal[np_unpack_indices(qbits, packed[pos:pos + nbytes], n)]
+        pos += nbytes
+    return out
+
+
+def np_dense64(X, W, bias=None) -> np.ndarray:
+    y = X.astype(np.float64) @ W.astype(np.float64).T
+    if bias is not None:
+        y = y + bias.astype(np.float64)
+    return y
+
+
+def np_rmsnorm64(x, gamma, eps=1e-6) -> np.ndarray:
+    x = x.astype(np.float64)
+    y = x / np.sqrt((x * x).mean(axis=-1, keepdims=True) + eps)
+    return y if gamma is None else y * gamma.astype(np.float64)
+
+
+def np_cmul64(x, rot) -> np.ndarray:
+    """x [S,H,D], rot [S,D] interleaved (cos, sin) -> float64 [S,H,D]."""
+    x = x.astype(np.float64)
+    r = rot.astype(np.float64)[:, None, :]
+    xc = x[..., 0::2] + 1j * x[..., 1::2]
+    rc = r[..., 0::2] + 1j * r[..., 1::2]
+    yc = xc * rc
+    y = np.empty_like(x)
+    y[..., 0::2] = yc.real
+    y[..., 1::2] = yc.imag
+    return y
+
+
+def np_sdpa64(q, k, v, scale) -> np.ndarray:
+    """Brute-force float64 attention, [B,S,H,D] layout, GQA by head grouping."""
+    q = q.astype(np.float64)
+    k = k.astype(np.float64)
+    v = v.astype(np.float64)
+    B, Sq, Hq, D = q.shape
+    Hk = k.shape[2]
+    g = Hq // Hk
+    o = np.zeros((B, Sq, Hq, D))
+    for b in range(B):
+        for h in range(Hq):
+            s = scale * (q[b, :, h] @ k[b, :, h // g].T)
+            s = s - s.max(axis=1, keepdims=True)
+            p = np.exp(s)
+            p /= p.sum(axis=1, keepdims=True)
+            o[b, :, h] = p @ v[b, :, h // g]
+    return o
+
+
+def err_stats(got, want):
+    """(max-abs, rel-RMS) of got vs want, both computed in float64."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    d = got - want
+    max_abs = float(np.abs(d).max()) if d.size else 0.0
+    den = float(np.sqrt((want * want).mean())) if d.size else 1.0
+    rel_rms = float(np.sqrt((d * d).mean()) / den) if den > 0 else float(np.sqrt((d * d).mean()))
+    return max_abs, rel_rms
+
+
+def synth_qx_weight(rng, N, K, qbits, nib, std=0.02):
+    """BASELINE-style synthetic palettized weight: per-block N(0, std) fp16
+    palettes and uniform indices.  Returns (packed uint8, palettes, idx)."""
+    count = N * K
+    nblocks = (count + nib - 1) // nib
+    palettes = (rng.standard_normal((nblocks, 1 << qbits)) * std).astype(np.float16)
+    idx = rng.integers(0, 1 << qbits, size=count, dtype=np.uint8)
+    return C.palettize_pack(qbits, nib, palettes, idx), palettes, idx
