@@ -1,0 +1,484 @@
+"""Host side of the MI355X transformer-block hot path.
+
+Mirrors the operator surface the reference's model builders use
+(`Dense`, `RMSNorm`, `Functional.cmul`, `ScaledDotProductAttention`,
+the rotary-table builders) on top of the C-ABI HIP library `libdthip.so`
+declared in `include/dt_hip.h`.  torch is used for device memory and streams
+only; every operator below runs a hand-written gfx950 kernel through ctypes
+and raises if the library is missing or a call fails.  There is no CPU path.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdthip.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+DT_OK, DT_INVALID, DT_NO_KERNEL, DT_OOM = 0, -1, -2, -3
+_STATUS = {0: "DT_OK", -1: "DT_INVALID", -2: "DT_NO_KERNEL", -3: "DT_OOM"}
+
+# every symbol include/dt_hip.h declares
+ABI_SYMBOLS = (
+    "dt_version",
+    "dt_init",
+    "dt_qx_bytes",
+    "dt_depalettize_f16",
+    "dt_dense_qx_f16",
+    "dt_qk_norm_rope_f16",
+    "dt_sdpa_f16",
+    "dt_sdpa_workspace_bytes",
+)
+
+
+class DtError(RuntimeError):
+    def __init__(self, fn: str, status: int):
+        super().__init__(f"{fn} failed: {_STATUS.get(status, status)}")
+        self.status = status
+
+
+class _QxWeight(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("qbits", ctypes.c_int32), ("nib", ctypes.c_int32), ("count", ctypes.c_int64)]
+
+
+class _View4(ctypes.Structure):
+    _fields_ = [("ptr", ctypes.c_void_p), ("stride_b", ctypes.c_int64), ("stride_s", ctypes.c_int64),
+                ("stride_h", ctypes.c_int64)]
+
+
+class _Segment(ctypes.Structure):
+    _fields_ = [("view", _View4), ("len", ctypes.c_int64), ("gamma", ctypes.c_void_p)]
+
+
+def build(verbose: bool = False) -> str:
+    """Compile libdthip.so for gfx950 with the Makefile under csrc/ (always recompiles)."""
+    cmd = ["make", "-C", CSRC, "-B", "-j8"]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if verbose or res.returncode != 0:
+        print(res.stdout)
+    if res.returncode != 0:
+        raise RuntimeError("building libdthip.so failed")
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    """The loaded C-ABI library.  Raises if it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with __graft_entry__.build() or `make -C {CSRC}`; "
+                "this package has no CPU or PyTorch fallback"
+            )
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i32, i64, f32 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float
+        L.dt_version.restype = ctypes.c_char_p
+        L.dt_version.argtypes = []
+        L.dt_init.restype = i32
+        L.dt_init.argtypes = [ctypes.c_int]
+        L.dt_qx_bytes.restype = i64
+        L.dt_qx_bytes.argtypes = [i32, i32, i64]
+        L.dt_depalettize_f16.restype = i32
+        L.dt_depalettize_f16.argtypes = [vp, ctypes.POINTER(_QxWeight), vp]
+        L.dt_dense_qx_f16.restype = i32
+        L.dt_dense_qx_f16.argtypes = [vp, i64, i64, vp, i64, ctypes.POINTER(_QxWeight), i32,
+                                      ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(i64), ctypes.c_uint32]
+        L.dt_qk_norm_rope_f16.restype = i32
+        L.dt_qk_norm_rope_f16.argtypes = [vp, _View4, i32, i64, i32, i32, vp, f32, i32, vp, i64, f32]
+        L.dt_sdpa_f16.restype = i32
+        L.dt_sdpa_f16.argtypes = [vp, i32, i32, i32, i32, i32, ctypes.POINTER(_Segment), i32,
+                                  ctypes.POINTER(_Segment), ctypes.POINTER(_Segment), vp, vp, f32, _View4, f32,
+                                  vp, vp, vp, ctypes.c_size_t]
+        L.dt_sdpa_workspace_bytes.restype = ctypes.c_size_t
+        L.dt_sdpa_workspace_bytes.argtypes = [i32, i32, i32, i32, i64, i64, i32, i32]
+        _lib = L
+    return _lib
+
+
+def _check(fn: str, status: int):
+    if status != DT_OK:
+        raise DtError(fn, status)
+
+
+def _torch():
+    import torch
+
+    return torch
+
+
+def _stream_ptr(stream=None):
+    torch = _torch()
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return ctypes.c_void_p(s.cuda_stream)
+
+
+def _f16_cuda(t, name):
+    torch = _torch()
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float16):
+        raise TypeError(f"{name} must be a CUDA float16 tensor")
+    return t
+
+
+# --------------------------------------------------------------------------
+# palettized weights
+# --------------------------------------------------------------------------
+
+# Elements per palette block for each codec.  Derived from the shipped model
+# sizes (about 0.25 bit/weight of palette overhead for q6p/q8p, 0.5 for
+# q4p/q5p); the library itself takes (qbits, nib) at run time.
+CODEC = {"q4p": (4, 512), "q5p": (5, 1024), "q6p": (6, 4096), "q7p": (7, 8192), "q8p": (8, 16384)}
+
+
+def qx_bytes(qbits: int, nib: int, count: int) -> int:
+    return int(lib().dt_qx_bytes(qbits, nib, count))
+
+
+def pack_indices(qbits: int, idx: np.ndarray) -> np.ndarray:
+    """MSB-first bit stream of `qbits`-wide indices (host-side producer of the format).
+    Eight indices always fill exactly `qbits` bytes: build each group as one 64-bit
+    big-endian number and cut it into bytes."""
+    idx = np.asarray(idx, dtype=np.uint8).reshape(-1)
+    n = idx.size
+    nbytes = (n * qbits + 7) // 8
+    if qbits == 8:
+        return idx.copy()
+    groups = (n + 7) // 8
+    padded = np.zeros(groups * 8, dtype=np.uint64)
+    padded[:n] = idx & ((1 << qbits) - 1)
+    padded = padded.reshape(groups, 8)
+    val = np.zeros(groups, dtype=np.uint64)
+    for j in range(8):
+        val |= padded[:, j] << np.uint64(qbits * (7 - j))
+    out = np.empty((groups, qbits), dtype=np.uint8)
+    for i in range(qbits):
+        out[:, i] = (val >> np.uint64(8 * (qbits - 1 - i))).astype(np.uint8)
+    return out.reshape(-1)[:nbytes].copy()
+
+
+def pack_qx(qbits: int, nib: int, palettes: np.ndarray, idx: np.ndarray) -> np.ndarray:
+    """Packed buffer from per-block fp16 palettes [nblocks, 2^q] and indices [count]."""
+    idx = np.asarray(idx, dtype=np.uint8).reshape(-1)
+    palettes = np.ascontiguousarray(palettes, dtype=np.float16)
+    count = idx.size
+    nblocks = (count + nib - 1) // nib
+    if palettes.shape != (nblocks, 1 << qbits):
+        raise ValueError(f"palettes must be [{nblocks}, {1 << qbits}]")
+    full = count // nib
+    pal_bytes = 2 << qbits
+    blk_bytes = nib * qbits // 8 if (nib * qbits) % 8 == 0 else None
+    chunks = []
+    if blk_bytes is not None and full > 0:
+        # all full blocks at once
+        packed = pack_indices(qbits, idx[: full * nib]).reshape(full, blk_bytes)
+        body = np.empty((full, pal_bytes + blk_bytes), dtype=np.uint8)
+        body[:, :pal_bytes] = palettes[:full].view(np.uint8).reshape(full, pal_bytes)
+        body[:, pal_bytes:] = packed
+        chunks.append(body.reshape(-1))
+        start = full
+    else:
+        start = 0
+    for b in range(start, nblocks):
+        chunks.append(palettes[b].view(np.uint8).reshape(-1))
+        chunks.append(pack_indices(qbits, idx[b * nib:(b + 1) * nib]))
+    return np.concatenate(chunks) if chunks else np.zeros(0, np.uint8)
+
+
+@dataclass
+class QxTensor:
+    """A weight as `store.read(codec: [.jit, .q?p])` leaves it: packed, on the device.
+
+    qbits == 16 means a plain fp16 [out, in] tensor (data is then a float16 tensor)."""
+
+    data: "object"  # torch uint8 (packed) or float16 tensor on the GPU
+    qbits: int
+    nib: int
+    shape: tuple  # (out, in)
+
+    @property
+    def count(self) -> int:
+        return int(self.shape[0]) * int(self.shape[1])
+
+    def _c(self) -> _QxWeight:
+        return _QxWeight(self.data.data_ptr(), self.qbits, self.nib, self.count)
+
+    @staticmethod
+    def from_packed(packed: np.ndarray, qbits: int, nib: int, shape, device="cuda") -> "QxTensor":
+        torch = _torch()
+        want = qx_bytes(qbits, nib, int(shape[0]) * int(shape[1]))
+        packed = np.ascontiguousarray(packed, dtype=np.uint8)
+        if packed.size != want:
+            raise ValueError(f"packed buffer has {packed.size} bytes, layout needs {want}")
+        # pad so the device buffer is a whole number of dwords
+        buf = np.zeros((packed.size + 15) // 16 * 16, dtype=np.uint8)
+        buf[: packed.size] = packed
+        return QxTensor(torch.from_numpy(buf).to(device), qbits, nib, (int(shape[0]), int(shape[1])))
+
+    @staticmethod
+    def from_f16(w, device="cuda") -> "QxTensor":
+        torch = _torch()
+        if isinstance(w, np.ndarray):
+            w = torch.from_numpy(np.ascontiguousarray(w, dtype=np.float16))
+        w = w.to(device).contiguous()
+        return QxTensor(w, 16, 0, tuple(w.shape))
+
+    def dequantize(self, stream=None):
+        """fp16 [out, in] tensor (K0): what a CPU read of the same key followed by Tensor<Float16>(from:) holds."""
+        torch = _torch()
+        if self.qbits == 16:
+            return self.data.clone()
+        out = torch.empty(self.shape, dtype=torch.float16, device=self.data.device)
+        w = self._c()
+        _check("dt_depalettize_f16", lib().dt_depalettize_f16(_stream_ptr(stream), ctypes.byref(w), out.data_ptr()))
+        return out
+
+
+# --------------------------------------------------------------------------
+# operators (names and argument meaning follow the reference's Model DSL)
+# --------------------------------------------------------------------------
+
+class GEMMFlag:
+    Float16 = 1
+    Float32 = 2
+
+
+def dense_multi(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]], outs=None, flags: int = 0,
+                stream=None):
+    """Several Dense ops that share the input, one launch (x_q / x_k / x_v)."""
+    torch = _torch()
+    _f16_cuda(x, "x")
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    n = len(weights)
+    W = (_QxWeight * n)(*[w._c() for w in weights])
+    for w in weights:
+        if w.shape[1] != K:
+            raise ValueError(f"weight {w.shape} does not match input width {K}")
+    if outs is None:
+        outs = [torch.empty((M, w.shape[0]), dtype=torch.float16, device=x.device) for w in weights]
+    vp = ctypes.c_void_p
+    B = (vp * n)(*[None if b is None else _f16_cuda(b, "bias").data_ptr() for b in biases])
+    Y = (vp * n)(*[o.data_ptr() for o in outs])
+    LDY = (ctypes.c_int64 * n)(*[o.stride(0) for o in outs])
+    st = lib().dt_dense_qx_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, flags)
+    _check("dt_dense_qx_f16", st)
+    lead = tuple(x.shape[:-1])
+    return [o.reshape(lead + (o.shape[-1],)) if o.shape[0] == M and o.is_contiguous() else o for o in outs]
+
+
+class Dense:
+    """Dense(count:noBias:flags:name:) -- y = x W^T + b with W [count, in] (Models/Flux1.swift:161-176)."""
+
+    def __init__(self, count: int, noBias: bool = False, flags: int = 0, name: str = ""):
+        self.count, self.noBias, self.flags, self.name = count, noBias, flags, name
+        self.weight: Optional[QxTensor] = None
+        self.bias = None
+
+    def __call__(self, x, stream=None):
+        if self.weight is None:
+            raise RuntimeError(f"Dense {self.name!r}: weight not loaded")
+        if self.weight.shape[0] != self.count:
+            raise ValueError(f"Dense {self.name!r}: weight has {self.weight.shape[0]} rows, count is {self.count}")
+        b = None if self.noBias else self.bias
+        return dense_multi(x, [self.weight], [b], flags=self.flags, stream=stream)[0]
+
+
+def _view4(t) -> _View4:
+    if t.dim() != 4 or t.stride(3) != 1:
+        raise ValueError("expected a [B, S, H, D] tensor with contiguous D")
+    return _View4(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def qk_norm_rope_(x, gamma=None, eps: float = 1e-6, norm_per_head: bool = True, rot=None, rot_pos0: int = 0,
+                  post_scale: float = 1.0, stream=None):
+    """In place on [B, S, H, D]: RMSNorm (per head, or over the whole row), then cmul with `rot`, then a scale."""
+    _f16_cuda(x, "x")
+    B, S, H, D = x.shape
+    if rot is not None:
+        _f16_cuda(rot, "rot")
+        if rot.dim() != 2 or rot.shape[1] != D or not rot.is_contiguous() or rot.shape[0] < rot_pos0 + S:
+            raise ValueError("rot must be a contiguous [>= rot_pos0 + S, D] table")
+    if gamma is not None:
+        _f16_cuda(gamma, "gamma")
+        want = D if norm_per_head else H * D
+        if gamma.numel() != want or not gamma.is_contiguous():
+            raise ValueError(f"gamma must hold {want} elements")
+    st = lib().dt_qk_norm_rope_f16(
+        _stream_ptr(stream), _view4(x), B, S, H, D, None if gamma is None else gamma.data_ptr(), eps,
+        1 if norm_per_head else 0, None if rot is None else rot.data_ptr(), rot_pos0, post_scale)
+    _check("dt_qk_norm_rope_f16", st)
+    return x
+
+
+class RMSNorm:
+    """RMSNorm(epsilon:axis:name:) on [B, S, H, D] (axis [3], per head) or [B, S, C] (axis [2], whole row)."""
+
+    def __init__(self, epsilon: float, axis: Sequence[int], name: str = ""):
+        self.epsilon, self.axis, self.name = epsilon, list(axis), name
+        self.weight = None
+
+    def __call__(self, x, stream=None):
+        y = x.clone()
+        if x.dim() == 4 and self.axis == [3]:
+            return qk_norm_rope_(y, self.weight, self.epsilon, True, stream=stream)
+        if x.dim() == 3 and self.axis == [2]:
+            qk_norm_rope_(_as_heads(y), self.weight, self.epsilon, False, stream=stream)
+            return y
+        raise DtError("RMSNorm", DT_NO_KERNEL)
+
+
+def _as_heads(y):
+    B, S, C = y.shape
+    for d in (128, 64, 32, 16, 8, 2):
+        if C % d == 0:
+            return y.view(B, S, C // d, d)
+    raise DtError("RMSNorm", DT_NO_KERNEL)
+
+
+class Functional:
+    @staticmethod
+    def cmul(left, right, stream=None):
+        """Complex multiply on adjacent pairs; `right` is the [1, S, 1, D] (or [S, D]) rotary table."""
+        y = left.clone()
+        rot = right.reshape(-1, right.shape[-1]).contiguous()
+        return qk_norm_rope_(y, None, 0.0, True, rot=rot, stream=stream)
+
+
+class ScaledDotProductAttention:
+    """ScaledDotProductAttention(scale:isCausal:hasAttentionMask:flags:multiHeadOutputProjectionFused:name:)
+    (Models/Flux1.swift:228-232, Models/UNet.swift:122-155).  Inputs [B, S, H, D]; returns [B, Sq, Hq, D], or
+    [B, Sq, Hq*D] when the unify-heads projection is fused (then `.weight` [HD, HD] fp16 and `.bias`)."""
+
+    def __init__(self, scale: float, isCausal: bool = False, hasAttentionMask: bool = False, flags: int = 0,
+                 multiHeadOutputProjectionFused: bool = False, name: str = ""):
+        if isCausal or hasAttentionMask:
+            raise DtError("ScaledDotProductAttention(isCausal/hasAttentionMask)", DT_NO_KERNEL)
+        self.scale, self.flags, self.fused, self.name = float(scale), flags, multiHeadOutputProjectionFused, name
+        self.weight = None
+        self.bias = None
+
+    def __call__(self, queries, keys, values, stream=None):
+        return sdpa_segments([queries], [keys], [values], self.scale,
+                             Wo=self.weight if self.fused else None, bo=self.bias if self.fused else None,
+                             stream=stream)
+
+
+def sdpa_segments(q_segs, k_segs, v_segs, scale, gamma_q=None, gamma_k=None, rot_q=None, rot_k=None,
+                  eps: float = 1e-6, Wo=None, bo=None, out=None, stream=None):
+    """Attention over a joint sequence given as segments (text || image without a concat).
+    gamma_q / gamma_k: per-segment per-head RMSNorm weights (or None); rot_*: [S, D] tables."""
+    torch = _torch()
+    L = lib()
+    for t in list(q_segs) + list(k_segs) + list(v_segs):
+        _f16_cuda(t, "q/k/v")
+    B, _, Hq, D = q_segs[0].shape
+    Hk = k_segs[0].shape[2]
+    Sq = sum(t.shape[1] for t in q_segs)
+    Skv = sum(t.shape[1] for t in k_segs)
+    nq, nk = len(q_segs), len(k_segs)
+    gq = gamma_q or [None] * nq
+    gk = gamma_k or [None] * nk
+
+    def segs(ts, gs):
+        arr = (_Segment * len(ts))()
+        for i, (t, g) in enumerate(zip(ts, gs)):
+            arr[i] = _Segment(_view4(t), t.shape[1], None if g is None else _f16_cuda(g, "gamma").data_ptr())
+        return arr
+
+    qa, ka, va = segs(q_segs, gq), segs(k_segs, gk), segs(v_segs, [None] * nk)
+    prep = any(g is not None for g in list(gq) + list(gk)) or rot_q is not None or rot_k is not None
+    fused = Wo is not None
+    if out is None:
+        shape = (B, Sq, Hq * D) if fused else (B, Sq, Hq, D)
+        out = torch.empty(shape, dtype=torch.float16, device=q_segs[0].device)
+    if fused:
+        ov = _View4(out.data_ptr(), out.stride(0), out.stride(1), 0)
+    else:
+        ov = _view4(out)
+    need = L.dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, int(prep), int(fused))
+    ws = torch.empty(max(need, 256) + 256, dtype=torch.uint8, device=out.device) if need else None
+    ws_ptr = None
+    if ws is not None:
+        ws_ptr = (ws.data_ptr() + 255) & ~255
+    st = L.dt_sdpa_f16(
+        _stream_ptr(stream), B, Hq, Hk, D, nq, qa, nk, ka, va,
+        None if rot_q is None else _f16_cuda(rot_q, "rot_q").data_ptr(),
+        None if rot_k is None else _f16_cuda(rot_k, "rot_k").data_ptr(),
+        eps, ov, scale, None if Wo is None else _f16_cuda(Wo, "Wo").data_ptr(),
+        None if bo is None else _f16_cuda(bo, "bo").data_ptr(), ws_ptr, need)
+    _check("dt_sdpa_f16", st)
+    return out
+
+
+# --------------------------------------------------------------------------
+# rotary tables (host side, as in the reference: computed on the CPU in double,
+# stored as float, cast to fp16 on upload)
+# --------------------------------------------------------------------------
+
+def _axis_table(pos: np.ndarray, dim: int) -> np.ndarray:
+    k = np.arange(dim // 2, dtype=np.float64)
+    theta = pos.astype(np.float64)[:, None] * 1.0 / np.power(10000.0, k * 2 / dim)
+    out = np.empty((pos.size, dim), dtype=np.float32)
+    out[:, 0::2] = np.cos(theta)
+    out[:, 1::2] = np.sin(theta)
+    return out
+
+
+def Flux1RotaryPositionEmbedding(height: int, width: int, tokenLength: int, referenceSizes=(), channels: int = 128):
+    """[tokenLength + height*width + sum(ref), channels] float32 table (Models/Flux1.swift:5-119), heads = 1."""
+    assert channels % 16 == 0
+    dim0, dim1 = channels // 8, channels * 7 // 16
+    pos0 = [np.zeros(tokenLength + height * width)]
+    ys, xs = np.divmod(np.arange(height * width), width)
+    pos1 = [np.zeros(tokenLength), ys]
+    pos2 = [np.zeros(tokenLength), xs]
+    h = w = 0
+    for (rh, rw) in referenceSizes:
+        hoff = woff = 0
+        if rh + h > rw + w:
+            woff = w
+        else:
+            hoff = h
+        ys, xs = np.divmod(np.arange(rh * rw), rw)
+        pos0.append(np.ones(rh * rw))
+        pos1.append(ys + hoff)
+        pos2.append(xs + woff)
+        h, w = max(h, rh + hoff), max(w, rw + woff)
+    p0, p1, p2 = (np.concatenate(p) for p in (pos0, pos1, pos2))
+    return np.concatenate([_axis_table(p0, dim0), _axis_table(p1, dim1), _axis_table(p2, dim1)], axis=1)
+
+
+def WanRotaryPositionEmbedding(height: int, width: int, time: int, channels: int = 128):
+    """[time*height*width, channels] float32 table (Models/Wan.swift:5-46), heads = 1."""
+    assert channels % 16 == 0
+    dim1 = (channels // 6) * 2
+    dim0 = channels - 2 * dim1
+    i = np.arange(time * height * width)
+    t, rem = np.divmod(i, height * width)
+    y, x = np.divmod(rem, width)
+    return np.concatenate([_axis_table(t, dim0), _axis_table(y, dim1), _axis_table(x, dim1)], axis=1)
+
+
+# --------------------------------------------------------------------------
+# work units (Models/InstructionCount/InstructionCount.swift:4-17)
+# --------------------------------------------------------------------------
+
+def DenseInstructionCount(rows: int, input: int, output: int) -> int:
+    assert rows >= 0 and input >= 0 and output >= 0
+    return rows * output * input
+
+
+def ScaledDotProductAttentionInstructionCount(batchSize, heads, headDimension, sequenceDimensionA,
+                                              sequenceDimensionB) -> int:
+    return batchSize * heads * (2 * headDimension + 5) * sequenceDimensionA * sequenceDimensionB

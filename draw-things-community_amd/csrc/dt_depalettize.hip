@@ -1,0 +1,92 @@
+// K0: depalettize a packed tensor to fp16 (bit-exact table lookup).
+// HBM-bound byte work: reads count*q/8 + palettes, writes 2*count bytes.
+#include "dt_common.h"
+#include "dt_layout.h"
+
+namespace dt {
+
+// One thread per 32-element granule (needs nib % 32 == 0 so that a granule
+// never straddles a block and always starts on a dword of the index stream).
+template <int Q>
+__global__ void __launch_bounds__(256) depalettize32_kernel(const uint8_t* __restrict__ packed, int nib,
+                                                          int64_t n_granules, uint16_t* __restrict__ out) {
+  int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (g >= n_granules) return;
+  const QxLayout l = make_layout(Q, nib);
+  int64_t e = g * 32;
+  int64_t b = e / nib;
+  int64_t r = e - b * nib;
+  const uint16_t* pal = reinterpret_cast<const uint16_t*>(packed + palette_offset(l, b));
+  const uint32_t* src = reinterpret_cast<const uint32_t*>(packed + index_byte_offset(l, b, r));
+  uint32_t raw[Q];
+#pragma unroll
+  for (int i = 0; i < Q; i++) raw[i] = src[i];
+  uint32_t idx[32];
+  unpack32<Q>(raw, idx);
+  uint32_t o[16];
+#pragma unroll
+  for (int j = 0; j < 16; j++) o[j] = (uint32_t)pal[idx[2 * j]] | ((uint32_t)pal[idx[2 * j + 1]] << 16);
+  uint16_t* dst = out + e;
+  if ((reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+    uint4_t* d4 = reinterpret_cast<uint4_t*>(dst);
+#pragma unroll
+    for (int j = 0; j < 4; j++) d4[j] = uint4_t{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
+  } else {
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+      dst[2 * j] = (uint16_t)o[j];
+      dst[2 * j + 1] = (uint16_t)(o[j] >> 16);
+    }
+  }
+}
+
+// One thread per element: any nib, ragged tails.
+__global__ void __launch_bounds__(256) depalettize1_kernel(const uint8_t* __restrict__ packed, int qbits, int nib,
+                                                         int64_t first, int64_t count,
+                                                         uint16_t* __restrict__ out) {
+  int64_t e = first + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= count) return;
+  const QxLayout l = make_layout(qbits, nib);
+  int64_t b = e / nib;
+  int64_t r = e - b * nib;
+  const uint16_t* pal = reinterpret_cast<const uint16_t*>(packed + palette_offset(l, b));
+  const uint8_t* idx = packed + palette_offset(l, b) + l.pal_bytes;
+  out[e] = pal[load_index(idx, r, qbits)];
+}
+
+}  // namespace dt
+
+DT_EXPORT dt_status dt_depalettize_f16(dt_stream stream, const dt_qx_weight* w, uint16_t* out) {
+  using namespace dt;
+  if (!w || w->count < 0) return DT_INVALID;
+  if (w->count == 0) return DT_OK;
+  if (!w->data || !out) return DT_INVALID;
+  if (w->qbits < 4 || w->qbits > 8 || w->nib <= 0) return DT_INVALID;
+  if ((reinterpret_cast<uintptr_t>(out) & 1) != 0) return DT_INVALID;
+  if (!device_ok()) return DT_NO_KERNEL;
+  hipStream_t s = as_stream(stream);
+  const uint8_t* packed = static_cast<const uint8_t*>(w->data);
+  int64_t done = 0;
+  if (w->nib % 32 == 0 && (reinterpret_cast<uintptr_t>(packed) & 3) == 0) {
+    int64_t ng = w->count / 32;
+    if (ng > 0) {
+      if ((ng + 255) / 256 > 0x7fffffff) return DT_NO_KERNEL;
+      dim3 grid((unsigned)((ng + 255) / 256));
+      switch (w->qbits) {
+        case 4: hipLaunchKernelGGL(depalettize32_kernel<4>, grid, dim3(256), 0, s, packed, w->nib, ng, out); break;
+        case 5: hipLaunchKernelGGL(depalettize32_kernel<5>, grid, dim3(256), 0, s, packed, w->nib, ng, out); break;
+        case 6: hipLaunchKernelGGL(depalettize32_kernel<6>, grid, dim3(256), 0, s, packed, w->nib, ng, out); break;
+        case 7: hipLaunchKernelGGL(depalettize32_kernel<7>, grid, dim3(256), 0, s, packed, w->nib, ng, out); break;
+        default: hipLaunchKernelGGL(depalettize32_kernel<8>, grid, dim3(256), 0, s, packed, w->nib, ng, out); break;
+      }
+      done = ng * 32;
+    }
+  }
+  if (done < w->count) {
+    int64_t rest = w->count - done;
+    if ((rest + 255) / 256 > 0x7fffffff) return DT_NO_KERNEL;
+    hipLaunchKernelGGL(depalettize1_kernel, dim3((unsigned)((rest + 255) / 256)), dim3(256), 0, s, packed, w->qbits,
+                       w->nib, done, w->count, out);
+  }
+  return launch_status();
+}

@@ -1,0 +1,199 @@
+// Host side of the attention entry point: validation, segment tables, the
+// optional norm/rotate staging pass and the optional fused output projection.
+#include "dt_common.h"
+#include "dt_qkprep.h"
+#include "dt_sdpa.h"
+
+namespace dt {
+
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+static bool view_ok(const dt_view4& v, int align_elems) {
+  if (!v.ptr) return false;
+  const uintptr_t mask = (uintptr_t)align_elems * 2 - 1;
+  if (reinterpret_cast<uintptr_t>(v.ptr) & mask) return false;
+  return v.stride_b % align_elems == 0 && v.stride_s % align_elems == 0 && v.stride_h % align_elems == 0;
+}
+
+}  // namespace dt
+
+DT_EXPORT size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int64_t Sq, int64_t Skv,
+                                         int32_t fused_prep, int32_t fused_out_proj) {
+  using namespace dt;
+  if (B <= 0 || Hq <= 0 || Hk <= 0 || D <= 0 || Sq <= 0 || Skv <= 0) return 0;
+  size_t bytes = 0;
+  if (fused_prep) {
+    bytes += align256((size_t)B * Sq * Hq * D * 2);
+    bytes += align256((size_t)B * Skv * Hk * D * 2);
+  }
+  if (fused_out_proj) bytes += align256((size_t)B * Sq * Hq * D * 2);
+  return bytes;
+}
+
+DT_EXPORT dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D, int32_t n_qseg,
+                                const dt_seq_segment* q_seg, int32_t n_kvseg, const dt_seq_segment* k_seg,
+                                const dt_seq_segment* v_seg, const uint16_t* rot_q, const uint16_t* rot_k, float eps,
+                                dt_view4 o, float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
+                                size_t workspace_bytes) {
+  using namespace dt;
+  if (B < 0 || Hq <= 0 || Hk <= 0 || D <= 0 || Hq % Hk != 0) return DT_INVALID;
+  if (n_qseg <= 0 || n_kvseg <= 0 || !q_seg || !k_seg || !v_seg) return DT_INVALID;
+  if (n_qseg > kMaxSeg || n_kvseg > kMaxSeg) return DT_NO_KERNEL;
+  if (D % 8 != 0 || D > 128) return DT_NO_KERNEL;
+  int64_t Sq = 0, Skv = 0;
+  bool prep = rot_q || rot_k;
+  for (int i = 0; i < n_qseg; i++) {
+    if (q_seg[i].len < 0) return DT_INVALID;
+    Sq += q_seg[i].len;
+    prep = prep || q_seg[i].gamma;
+  }
+  for (int i = 0; i < n_kvseg; i++) {
+    if (k_seg[i].len < 0 || k_seg[i].len != v_seg[i].len) return DT_INVALID;
+    Skv += k_seg[i].len;
+    prep = prep || k_seg[i].gamma;
+  }
+  if (B == 0 || Sq == 0) return DT_OK;
+  if (Skv == 0) return DT_INVALID;  // softmax over an empty set
+  for (int i = 0; i < n_qseg; i++)
+    if (q_seg[i].len > 0 && !view_ok(q_seg[i].view, 8)) return DT_INVALID;
+  for (int i = 0; i < n_kvseg; i++)
+    if (k_seg[i].len > 0 && (!view_ok(k_seg[i].view, 8) || !view_ok(v_seg[i].view, 8))) return DT_INVALID;
+  if (!o.ptr || (reinterpret_cast<uintptr_t>(o.ptr) & 7) || o.stride_b % 4 || o.stride_s % 4) return DT_INVALID;
+  if (!Wo && o.stride_h % 4) return DT_INVALID;
+  if (!device_ok()) return DT_NO_KERNEL;
+
+  const size_t need = dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, prep ? 1 : 0, Wo ? 1 : 0);
+  if (need > 0) {
+    if (!workspace || workspace_bytes < need) return DT_OOM;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return DT_INVALID;
+  }
+  hipStream_t s = as_stream(stream);
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+
+  SdpaArgs a = {};
+  a.B = B;
+  a.Hq = Hq;
+  a.Hk = Hk;
+  a.group = Hq / Hk;
+  a.D = D;
+  a.Sq = Sq;
+  a.Skv = Skv;
+  a.scale_log2e = scale * 1.44269504088896340736f;
+
+  if (prep) {
+    // RMSNorm -> cmul staged into contiguous copies; V is read in place.
+    uint16_t* qw = reinterpret_cast<uint16_t*>(ws);
+    ws += align256((size_t)B * Sq * Hq * D * 2);
+    uint16_t* kw = reinterpret_cast<uint16_t*>(ws);
+    ws += align256((size_t)B * Skv * Hk * D * 2);
+    for (int pass = 0; pass < 2; pass++) {
+      const dt_seq_segment* seg = pass == 0 ? q_seg : k_seg;
+      const int n = pass == 0 ? n_qseg : n_kvseg;
+      const int H = pass == 0 ? Hq : Hk;
+      const int64_t S = pass == 0 ? Sq : Skv;
+      uint16_t* dst = pass == 0 ? qw : kw;
+      const uint16_t* rot = pass == 0 ? rot_q : rot_k;
+      int64_t pos = 0;
+      for (int i = 0; i < n; i++) {
+        if (seg[i].len == 0) continue;
+        QkPrepArgs p;
+        p.src = static_cast<const uint16_t*>(seg[i].view.ptr);
+        p.src_sb = seg[i].view.stride_b;
+        p.src_ss = seg[i].view.stride_s;
+        p.src_sh = seg[i].view.stride_h;
+        p.dst = dst + pos * H * D;
+        p.dst_sb = S * H * D;
+        p.dst_ss = (int64_t)H * D;
+        p.dst_sh = D;
+        p.B = B;
+        p.S = seg[i].len;
+        p.H = H;
+        p.D = D;
+        p.gamma = seg[i].gamma;
+        p.eps = eps;
+        p.norm_per_head = 1;
+        p.rot = rot;
+        p.rot_pos0 = pos;
+        p.post_scale = 1.0f;
+        dt_status st = qk_prep_launch(s, p);
+        if (st != DT_OK) return st;
+        pos += seg[i].len;
+      }
+    }
+    a.n_qseg = 1;
+    a.q[0] = SdpaSeg{qw, Sq * Hq * D, (int64_t)Hq * D, D, 0};
+    a.n_kvseg = 1;
+    a.k[0] = SdpaSeg{kw, Skv * Hk * D, (int64_t)Hk * D, D, 0};
+    for (int i = 1; i < kMaxSeg; i++) {
+      a.q[i] = a.q[0];
+      a.k[i] = a.k[0];
+    }
+  } else {
+    int64_t pos = 0;
+    int n = 0;
+    for (int i = 0; i < n_qseg; i++) {
+      if (q_seg[i].len == 0) continue;
+      const dt_view4& v = q_seg[i].view;
+      a.q[n++] = SdpaSeg{static_cast<const uint16_t*>(v.ptr), v.stride_b, v.stride_s, v.stride_h, pos};
+      pos += q_seg[i].len;
+    }
+    a.n_qseg = n;
+    for (int i = n; i < kMaxSeg; i++) a.q[i] = a.q[0];
+    pos = 0;
+    n = 0;
+    for (int i = 0; i < n_kvseg; i++) {
+      if (k_seg[i].len == 0) continue;
+      const dt_view4& v = k_seg[i].view;
+      a.k[n++] = SdpaSeg{static_cast<const uint16_t*>(v.ptr), v.stride_b, v.stride_s, v.stride_h, pos};
+      pos += k_seg[i].len;
+    }
+    a.n_kvseg = n;
+    for (int i = n; i < kMaxSeg; i++) a.k[i] = a.k[0];
+  }
+  {
+    int64_t pos = 0;
+    int n = 0;
+    for (int i = 0; i < n_kvseg; i++) {
+      if (v_seg[i].len == 0) continue;
+      const dt_view4& v = v_seg[i].view;
+      a.v[n++] = SdpaSeg{static_cast<const uint16_t*>(v.ptr), v.stride_b, v.stride_s, v.stride_h, pos};
+      pos += v_seg[i].len;
+    }
+    for (int i = n; i < kMaxSeg; i++) a.v[i] = a.v[0];
+    if (prep && n > 1) {
+      // K was staged as one segment; the V segments keep their own table
+      a.n_kvseg = n;
+      for (int i = 1; i < n; i++) {
+        a.k[i] = a.k[0];
+        a.k[i].start = a.v[i].start;
+        a.k[i].ptr = a.k[0].ptr + a.v[i].start * a.k[0].ss;
+      }
+    }
+  }
+
+  if (Wo) {
+    uint16_t* ow = reinterpret_cast<uint16_t*>(ws);
+    a.o = ow;
+    a.o_sb = Sq * Hq * D;
+    a.o_ss = (int64_t)Hq * D;
+    a.o_sh = D;
+    dt_status st = sdpa_launch(s, a);
+    if (st != DT_OK) return st;
+    // unify-heads projection on the staged attention output, batch by batch
+    const int64_t HD = (int64_t)Hq * D;
+    dt_qx_weight w{Wo, 16, 0, HD * HD};
+    for (int b = 0; b < B; b++) {
+      const uint16_t* bias_arr[1] = {bo};
+      uint16_t* y_arr[1] = {static_cast<uint16_t*>(o.ptr) + b * o.stride_b};
+      const int64_t ldy_arr[1] = {o.stride_s};
+      st = dt_dense_qx_f16(stream, Sq, HD, ow + b * a.o_sb, HD, &w, 1, bias_arr, y_arr, ldy_arr, 0);
+      if (st != DT_OK) return st;
+    }
+    return DT_OK;
+  }
+  a.o = static_cast<uint16_t*>(o.ptr);
+  a.o_sb = o.stride_b;
+  a.o_ss = o.stride_s;
+  a.o_sh = o.stride_h;
+  return sdpa_launch(s, a);
+}

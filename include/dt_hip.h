@@ -1,0 +1,176 @@
+/*
+ * dt_hip.h -- C ABI of the MI355X (gfx950) transformer-block hot path:
+ * Dense over palettized weights and ScaledDotProductAttention, plus the two
+ * small ops fused around them (per-head / per-row RMSNorm and the RoPE cmul).
+ *
+ * Plain C, no C++ or framework types cross this boundary.  Every pointer is a
+ * DEVICE pointer borrowed for the duration of the enqueue (the call returns
+ * once the work is queued on `stream`; it never synchronises the stream).
+ * All entry points are re-entrant and stream-ordered; the library keeps no
+ * mutable global state apart from a once-per-process device query.
+ *
+ * Status codes mirror the values a ccv_nnc backend `exec` returns, so a shim
+ * can map DT_NO_KERNEL to "fall through to the next backend":
+ *    0  DT_OK          work enqueued
+ *   -1  DT_INVALID     bad shape / alignment / NULL pointer / unknown qbits
+ *   -2  DT_NO_KERNEL   valid request this library has no kernel for
+ *   -3  DT_OOM         workspace too small
+ *
+ * The operator surface this replaces is the one the reference's model
+ * builders call (reference paths relative to Libraries/SwiftDiffusion/Sources):
+ *   Dense(count:noBias:flags:name:)                 Models/Flux1.swift:161-176, 237-245
+ *   RMSNorm(epsilon:axis:name:)                     Models/Flux1.swift:165-182, Models/Wan.swift:87-91
+ *   Functional.cmul(left:right:)                    Models/Flux1.swift:187-188, Models/Wan.swift:93-94
+ *   ScaledDotProductAttention(scale:flags:multiHeadOutputProjectionFused:)
+ *                                                   Models/Flux1.swift:228-232, Models/UNet.swift:122-155
+ *   store.read(_, codec:[.q4p/.q5p/.q6p/.q8p, .jit]) Models/UNetProtocol.swift:2230-2233, 2370-2373
+ */
+#ifndef DT_HIP_H
+#define DT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int32_t dt_status;
+#define DT_OK 0
+#define DT_INVALID (-1)
+#define DT_NO_KERNEL (-2)
+#define DT_OOM (-3)
+
+/* A hipStream_t passed as an opaque pointer; NULL is the default stream. */
+typedef void* dt_stream;
+
+/*
+ * A weight as store.read(codec: [.jit, .q?p]) leaves it on the device
+ * (Models/UNetProtocol.swift:2230-2233): still palettized.
+ *   data  : packed buffer, 16-byte aligned
+ *   qbits : 4, 5, 6, 7 or 8 -> per block of `nib` elements (flattened row-major
+ *           [out, in] order), 2^qbits fp16 palette entries followed by that
+ *           block's indices bit-packed MSB-first;
+ *           16 -> plain fp16 [out, in] weight (nib ignored)
+ *   nib   : elements per palette block
+ *   count : number of elements = out * in
+ */
+typedef struct {
+  const void* data;
+  int32_t qbits;
+  int32_t nib;
+  int64_t count;
+} dt_qx_weight;
+
+/* [B, S, H, D] fp16 view, D contiguous; strides in elements. */
+typedef struct {
+  void* ptr;
+  int64_t stride_b;
+  int64_t stride_s;
+  int64_t stride_h;
+} dt_view4;
+
+/* One run of consecutive sequence positions.  A joint text||image sequence
+ * (Functional.concat(axis: 1, contextK, xK), Models/Flux1.swift:184-186) is
+ * passed as two segments instead of a materialised concatenation.
+ *   gamma : per-head RMSNorm weight [D] applied to this segment's rows before
+ *           attention (c_norm_q / x_norm_q differ per segment,
+ *           Models/Flux1.swift:165-182); NULL = no norm */
+typedef struct {
+  dt_view4 view;
+  int64_t len;
+  const uint16_t* gamma;
+} dt_seq_segment;
+
+/* Library identification; never NULL. */
+const char* dt_version(void);
+
+/* Checks that `device` is a gfx950 part and warms the per-process device
+ * query.  Optional: every entry point does the same check lazily.
+ * Returns DT_NO_KERNEL on any other architecture. */
+dt_status dt_init(int device);
+
+/* Bytes a palettized tensor of `count` elements occupies, palettes included;
+ * -1 for an unsupported (qbits, nib). */
+int64_t dt_qx_bytes(int32_t qbits, int32_t nib, int64_t count);
+
+/*
+ * out[i] = palette[i / nib][index[i]]  -- the tensor a CPU read of the same
+ * key yields (store.read(name, kind: .CPU, codec: [.q6p, .q8p, ...]) followed
+ * by Tensor<FloatType>(from:), LoRALoader.swift:317).  Bit-exact.
+ * out: `count` fp16 values, 2-byte aligned.
+ */
+dt_status dt_depalettize_f16(dt_stream stream, const dt_qx_weight* w, uint16_t* out);
+
+/*
+ * Dense: Y = X W^T (+ bias), X [M, K] fp16 with row stride ldx, each W_i
+ * [N_i, K] (N_i = count_i / K), Y_i [M, N_i] fp16 with row stride ldy[i];
+ * fp32 accumulation, one rounding to fp16.  n_weights > 1 runs several Dense
+ * ops that share X in one launch (x_q / x_k / x_v, Models/Flux1.swift:174-176).
+ * The palettized weight is unpacked and looked up on chip; no dequantized
+ * copy is written to memory.
+ *   bias  : array of n_weights pointers, entries may be NULL (noBias: true);
+ *           the array itself may be NULL when no weight has a bias
+ *   flags : bit 0 = caller allows fp16 accumulation (Functional.GEMMFlag
+ *           .Float16, Models/Flux1.swift:162); accepted and ignored
+ * The arrays W / bias / Y / ldy are HOST arrays of n_weights entries.
+ */
+dt_status dt_dense_qx_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,
+                          const dt_qx_weight* W, int32_t n_weights, const uint16_t* const* bias,
+                          uint16_t* const* Y, const int64_t* ldy, uint32_t flags);
+
+/*
+ * In place on a [B, S, H, D] view: optional RMSNorm, then optional RoPE.
+ *   gamma       : RMSNorm weight, [D] when norm_per_head != 0 (Flux:
+ *                 RMSNorm(axis: [3]), Models/Flux1.swift:165), [H*D] when 0
+ *                 (Wan: RMSNorm(axis: [2]) over the whole row before the head
+ *                 split, Models/Wan.swift:87-91; needs stride_h == D); NULL = skip
+ *   rot         : [>= rot_pos0 + S, D] fp16 table of interleaved (cos, sin)
+ *                 pairs, row stride D, broadcast over batch and heads
+ *                 (Functional.cmul, Models/Flux1.swift:187-188); NULL = skip
+ *   rot_pos0    : table row of this view's first position (a segment of a
+ *                 joint sequence starts at its offset in the joint order)
+ *   post_scale  : multiplies the result (Wan's .scale1 convention scales Q and
+ *                 K by D^-1/4, Models/Wan.swift:95-98); 1.0f = none
+ * Rounds to fp16 after the norm, after the rotation and after the scale, as
+ * the op-by-op graph does.
+ */
+dt_status dt_qk_norm_rope_f16(dt_stream stream, dt_view4 x, int32_t B, int64_t S, int32_t H,
+                              int32_t D, const uint16_t* gamma, float eps, int32_t norm_per_head,
+                              const uint16_t* rot, int64_t rot_pos0, float post_scale);
+
+/*
+ * O = softmax(scale * Q K^T) V per (batch, head); non-causal, no mask.
+ *   Q rows  : concatenation of n_qseg segments (each [B, len, Hq, D])
+ *   K/V rows: concatenation of n_kvseg segments (each [B, len, Hk, D]);
+ *             k_seg[i].len must equal v_seg[i].len; Hk divides Hq
+ *   rot_q / rot_k : optional RoPE tables [total rows, D] indexed by position
+ *             in the joint order; together with the segments' gamma this is
+ *             the fused form of RMSNorm -> concat -> cmul -> attention
+ *             (Models/Flux1.swift:165-188, 228-232); v_seg[i].gamma is ignored
+ *   o       : [B, total Q rows, Hq, D]; when Wo != NULL the unify-heads
+ *             projection is fused (multiHeadOutputProjectionFused: true,
+ *             Models/UNet.swift:143-155): o is then [B, Sq, Hq*D] written with
+ *             o.stride_s as row stride (stride_h unused), Wo fp16 [Hq*D, Hq*D]
+ *             in [out, in] order, bo [Hq*D] or NULL
+ *   workspace : device scratch of at least dt_sdpa_workspace_bytes(...) bytes,
+ *             256-byte aligned; may be NULL when that function returns 0
+ * D in {40, 64, 128} (any D <= 128 that is a multiple of 8).
+ */
+dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D,
+                      int32_t n_qseg, const dt_seq_segment* q_seg, int32_t n_kvseg,
+                      const dt_seq_segment* k_seg, const dt_seq_segment* v_seg,
+                      const uint16_t* rot_q, const uint16_t* rot_k, float eps, dt_view4 o,
+                      float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
+                      size_t workspace_bytes);
+
+/* Scratch dt_sdpa_f16 needs: room for normalised / rotated copies of Q and K
+ * when `fused_prep` != 0 (any gamma or rot given) and for the attention output
+ * when `fused_out_proj` != 0. */
+size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int64_t Sq,
+                               int64_t Skv, int32_t fused_prep, int32_t fused_out_proj);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DT_HIP_H */

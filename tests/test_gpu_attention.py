@@ -1,0 +1,268 @@
+"""GPU parity: RMSNorm + RoPE (K2) and ScaledDotProductAttention (K3) against the CPU oracle, through the C ABI.
+
+Bar for attention outputs: max-abs <= 2e-2, rel-RMS <= 1e-3.  The norm / rotate pass rounds where the oracle
+rounds, so it is held to one fp16 ulp."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, REL_RMS = 2e-2, 1e-3
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+
+    assert torch.cuda.is_available()
+    return torch
+
+
+def to_dev(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def f16(a):
+    return np.asarray(a, dtype=np.float16)
+
+
+def ulp_close(got, want, ulps=1):
+    got = got.astype(np.float64)
+    want = want.astype(np.float64)
+    tol = ulps * (np.abs(want) * 2.0 ** -10 + 2.0 ** -24)
+    return np.all(np.abs(got - want) <= tol)
+
+
+# ------------------------------------------------------------------ K2
+
+@pytest.mark.parametrize("D,H", [(128, 24), (64, 8), (40, 8)])
+def test_rmsnorm_per_head(dthip, oracle, torch_cuda, D, H):
+    torch = torch_cuda
+    rng = np.random.default_rng(D)
+    x = f16(rng.standard_normal((2, 37, H, D)))
+    g = f16(1 + 0.02 * rng.standard_normal(D))
+    n = dthip.RMSNorm(epsilon=1e-6, axis=[3], name="x_norm_q")
+    n.weight = to_dev(torch, g)
+    print("rmsnorm head", D, H, flush=True)
+    got = n(to_dev(torch, x)).cpu().numpy()
+    assert ulp_close(got, oracle.C.rmsnorm(x, g, 1e-6))
+
+
+def test_rmsnorm_whole_row(dthip, oracle, torch_cuda):
+    """Wan: RMSNorm(axis: [2]) over the 5120-wide row before the head split."""
+    torch = torch_cuda
+    rng = np.random.default_rng(1)
+    x = f16(rng.standard_normal((1, 50, 5120)))
+    g = f16(1 + 0.02 * rng.standard_normal(5120))
+    n = dthip.RMSNorm(epsilon=1e-6, axis=[2], name="x_norm_k")
+    n.weight = to_dev(torch, g)
+    print("rmsnorm row", flush=True)
+    got = n(to_dev(torch, x)).cpu().numpy()
+    assert ulp_close(got, oracle.C.rmsnorm(x, g, 1e-6))
+
+
+def test_cmul_rope(dthip, oracle, torch_cuda):
+    torch = torch_cuda
+    rng = np.random.default_rng(2)
+    h, w, t = 6, 5, 7
+    S = t + h * w
+    x = f16(rng.standard_normal((1, S, 4, 128)))
+    rot = f16(dthip.Flux1RotaryPositionEmbedding(h, w, t, channels=128))
+    print("cmul", flush=True)
+    got = dthip.Functional.cmul(to_dev(torch, x), to_dev(torch, rot.reshape(1, S, 1, 128))).cpu().numpy()
+    want = oracle.C.cmul(x[0], rot)
+    assert np.array_equal(got[0].view(np.uint16), want.view(np.uint16))
+    # text rows (theta = 0) pass through unchanged
+    assert np.array_equal(got[0, :t], x[0, :t])
+
+
+def test_norm_rope_scale_in_place_on_strided_view(dthip, oracle, torch_cuda):
+    """Flux per-head norm + RoPE at a joint-sequence offset, then Wan's D^-1/4 scale, on a view into a wider buffer."""
+    torch = torch_cuda
+    rng = np.random.default_rng(3)
+    B, S, H, D, pos0 = 2, 33, 3, 128, 9
+    buf = f16(rng.standard_normal((B, S, 3 * H * D)))
+    g = f16(1 + 0.02 * rng.standard_normal(D))
+    rot = f16(dthip.Flux1RotaryPositionEmbedding(7, 6, pos0, channels=D))
+    dev = to_dev(torch, buf)
+    view = dev[:, :, H * D:2 * H * D].unflatten(2, (H, D))  # the K third of a fused QKV buffer
+    s4 = float(D) ** -0.25
+    print("norm rope in place", flush=True)
+    dthip.qk_norm_rope_(view, to_dev(torch, g), 1e-6, True, rot=to_dev(torch, rot), rot_pos0=pos0, post_scale=s4)
+    got = dev.cpu().numpy()
+    x = np.ascontiguousarray(buf[:, :, H * D:2 * H * D]).reshape(B, S, H, D)
+    want = np.stack([oracle.C.cmul(oracle.C.rmsnorm(x[b], g, 1e-6), rot[pos0:pos0 + S]) for b in range(B)])
+    want = f16(want.astype(np.float32) * np.float32(s4))
+    assert ulp_close(got[:, :, H * D:2 * H * D].reshape(B, S, H, D), want)
+    # everything outside the view is untouched
+    assert np.array_equal(got[:, :, :H * D], buf[:, :, :H * D]) and np.array_equal(got[:, :, 2 * H * D:], buf[:, :, 2 * H * D:])
+
+
+# ------------------------------------------------------------------ K3
+
+def rand_qkv(rng, B, Sq, Skv, Hq, Hk, D):
+    return (f16(rng.standard_normal((B, Sq, Hq, D))), f16(rng.standard_normal((B, Skv, Hk, D))),
+            f16(rng.standard_normal((B, Skv, Hk, D))))
+
+
+SDPA_CASES = [
+    # B, Sq, Skv, Hq, Hk, D
+    (1, 128, 64, 2, 2, 128),
+    (1, 256, 256, 2, 2, 128),
+    (2, 200, 333, 3, 3, 128),     # ragged both ways
+    (1, 1, 1, 1, 1, 128),         # single query, single key
+    (1, 70, 77, 8, 8, 40),        # SD1.5 cross-attention shape (D = 40, 77 keys)
+    (2, 300, 300, 8, 8, 40),      # SD1.5 self-attention (reduced sequence)
+    (1, 130, 190, 4, 2, 64),      # grouped heads, D = 64
+    (1, 2100, 150, 2, 1, 128),    # long query side -> 64-row-per-wave kernel, grouped heads
+    (1, 2050, 257, 2, 2, 64),
+]
+
+
+@pytest.mark.parametrize("B,Sq,Skv,Hq,Hk,D", SDPA_CASES)
+def test_sdpa_vs_oracle(dthip, oracle, torch_cuda, B, Sq, Skv, Hq, Hk, D):
+    torch = torch_cuda
+    rng = np.random.default_rng(B * 1000 + Sq + Skv + D)
+    q, k, v = rand_qkv(rng, B, Sq, Skv, Hq, Hk, D)
+    scale = 1 / np.sqrt(D)
+    print("sdpa", B, Sq, Skv, Hq, Hk, D, flush=True)
+    op = dthip.ScaledDotProductAttention(scale=scale, flags=dthip.GEMMFlag.Float16)
+    got = op(to_dev(torch, q), to_dev(torch, k), to_dev(torch, v)).cpu().numpy()
+    want = oracle.C.sdpa(q, k, v, scale)
+    mx, rr = oracle.err_stats(got, want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+def test_sdpa_invariants(dthip, oracle, torch_cuda):
+    torch = torch_cuda
+    rng = np.random.default_rng(5)
+    B, Sq, Skv, H, D = 1, 150, 210, 2, 128
+    q, k, v = rand_qkv(rng, B, Sq, Skv, H, H, D)
+    op = dthip.ScaledDotProductAttention(scale=1 / np.sqrt(D))
+    qd, kd, vd = (to_dev(torch, t) for t in (q, k, v))
+    print("sdpa invariants", flush=True)
+    base = op(qd, kd, vd).cpu().numpy()
+    # constant V -> O is that constant
+    vc = np.broadcast_to(f16(rng.standard_normal((1, 1, H, D))), v.shape).copy()
+    oc = op(qd, kd, to_dev(torch, vc)).cpu().numpy()
+    assert np.max(np.abs(oc.astype(np.float64) - vc[:, :1].astype(np.float64))) <= 2e-3
+    # joint permutation of K / V rows
+    perm = rng.permutation(Skv)
+    op_ = op(qd, to_dev(torch, k[:, perm]), to_dev(torch, v[:, perm])).cpu().numpy()
+    assert np.max(np.abs(op_.astype(np.float64) - base.astype(np.float64))) <= 4e-3
+    # .scale1 convention: Q, K pre-multiplied by D^-1/4 and scale 1  ==  .scaleMerged within tolerance
+    s4 = np.float16(D ** -0.25)
+    o1 = dthip.ScaledDotProductAttention(scale=1.0)(to_dev(torch, f16(q * s4)), to_dev(torch, f16(k * s4)), vd)
+    mx, rr = oracle.err_stats(o1.cpu().numpy(), base)
+    assert mx <= MAX_ABS and rr <= 5e-3
+    # large logits stay finite (running max is subtracted before the exponential)
+    big = op(to_dev(torch, f16(q * 30)), to_dev(torch, f16(k * 30)), vd).cpu().numpy()
+    assert np.all(np.isfinite(big))
+    mx, rr = oracle.err_stats(big, oracle.C.sdpa(f16(q * 30), f16(k * 30), v, 1 / np.sqrt(D)))
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+def test_sdpa_segments_equal_concat_and_strided_views(dthip, oracle, torch_cuda):
+    """text || image passed as two segments == the concatenated call; Q/K/V are slices of one fused QKV buffer."""
+    torch = torch_cuda
+    rng = np.random.default_rng(6)
+    B, T, HW, H, D = 1, 70, 200, 3, 128
+    ctx = f16(rng.standard_normal((B, T, 3, H, D)))      # fused [q|k|v] buffers: stride_s = 3*H*D
+    img = f16(rng.standard_normal((B, HW, 3, H, D)))
+    cd, xd = to_dev(torch, ctx), to_dev(torch, img)
+    scale = 1 / np.sqrt(D)
+    print("sdpa segments", flush=True)
+    got = dthip.sdpa_segments([cd[:, :, 0], xd[:, :, 0]], [cd[:, :, 1], xd[:, :, 1]], [cd[:, :, 2], xd[:, :, 2]],
+                              scale).cpu().numpy()
+    q = np.concatenate([ctx[:, :, 0], img[:, :, 0]], axis=1)
+    k = np.concatenate([ctx[:, :, 1], img[:, :, 1]], axis=1)
+    v = np.concatenate([ctx[:, :, 2], img[:, :, 2]], axis=1)
+    want = oracle.C.sdpa(q, k, v, scale)
+    mx, rr = oracle.err_stats(got, want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+    cat = dthip.ScaledDotProductAttention(scale=scale)(to_dev(torch, q), to_dev(torch, k), to_dev(torch, v))
+    assert np.array_equal(cat.cpu().numpy().view(np.uint16), got.view(np.uint16))
+
+
+def test_sdpa_fused_norm_rope_joint(dthip, oracle, torch_cuda):
+    """The Flux joint block's attention input stage fused into the call: per-segment per-head RMSNorm
+    (c_norm_* / x_norm_*), RoPE over the joint order, then attention."""
+    torch = torch_cuda
+    rng = np.random.default_rng(7)
+    B, T, h, w, H, D = 1, 40, 12, 10, 2, 128
+    HW = h * w
+    segs = {n: (f16(rng.standard_normal((B, T, H, D))), f16(rng.standard_normal((B, HW, H, D)))) for n in "qkv"}
+    gam = {n: (f16(1 + 0.05 * rng.standard_normal(D)), f16(1 + 0.05 * rng.standard_normal(D))) for n in "qk"}
+    rot = f16(dthip.Flux1RotaryPositionEmbedding(h, w, T, channels=D))
+    scale = 1 / np.sqrt(D)
+    dev = lambda a: to_dev(torch, a)
+    print("sdpa fused prep", flush=True)
+    got = dthip.sdpa_segments(
+        [dev(t) for t in segs["q"]], [dev(t) for t in segs["k"]], [dev(t) for t in segs["v"]], scale,
+        gamma_q=[dev(g) for g in gam["q"]], gamma_k=[dev(g) for g in gam["k"]], rot_q=dev(rot), rot_k=dev(rot),
+    ).cpu().numpy()
+
+    def prep(n):
+        parts = [oracle.C.rmsnorm(segs[n][i][0], gam[n][i], 1e-6) for i in range(2)]
+        return oracle.C.cmul(np.concatenate(parts, axis=0), rot)[None]
+
+    want = oracle.C.sdpa(prep("q"), prep("k"), np.concatenate(segs["v"], axis=1), scale)
+    mx, rr = oracle.err_stats(got, want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+def test_sdpa_fused_output_projection(dthip, oracle, torch_cuda):
+    """SD1.5: multiHeadOutputProjectionFused -- the op owns W_o [HD, HD] and b_o and returns [B, S, HD]."""
+    torch = torch_cuda
+    rng = np.random.default_rng(8)
+    B, Sq, Skv, H, D = 2, 200, 77, 8, 40
+    q, k, v = rand_qkv(rng, B, Sq, Skv, H, H, D)
+    Wo = f16(rng.standard_normal((H * D, H * D)) * 0.05)
+    bo = f16(rng.standard_normal(H * D) * 0.05)
+    op = dthip.ScaledDotProductAttention(scale=1 / np.sqrt(D), multiHeadOutputProjectionFused=True)
+    op.weight, op.bias = to_dev(torch, Wo), to_dev(torch, bo)
+    print("sdpa fused out-proj", flush=True)
+    got = op(to_dev(torch, q), to_dev(torch, k), to_dev(torch, v)).cpu().numpy()
+    att = oracle.C.sdpa(q, k, v, 1 / np.sqrt(D)).reshape(B * Sq, H * D)
+    want = oracle.C.dense(att, Wo, bo).reshape(B, Sq, H * D)
+    mx, rr = oracle.err_stats(got, want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+def test_sdpa_rejects_bad_arguments(dthip, torch_cuda):
+    torch = torch_cuda
+    z = lambda *s: torch.zeros(s, dtype=torch.float16, device="cuda")
+    with pytest.raises(dthip.DtError) as e:
+        dthip.sdpa_segments([z(1, 8, 3, 64)], [z(1, 8, 2, 64)], [z(1, 8, 2, 64)], 1.0)  # 2 does not divide 3
+    assert e.value.status == dthip.DT_INVALID
+    with pytest.raises(dthip.DtError) as e:
+        dthip.sdpa_segments([z(1, 8, 2, 136)], [z(1, 8, 2, 136)], [z(1, 8, 2, 136)], 1.0)  # D > 128
+    assert e.value.status == dthip.DT_NO_KERNEL
+    with pytest.raises(dthip.DtError) as e:
+        dthip.sdpa_segments([z(1, 8, 2, 64)], [z(1, 0, 2, 64)], [z(1, 0, 2, 64)], 1.0)  # no keys
+    assert e.value.status == dthip.DT_INVALID
+    assert dthip.sdpa_segments([z(1, 0, 2, 64)], [z(1, 4, 2, 64)], [z(1, 4, 2, 64)], 1.0).shape == (1, 0, 2, 64)
+
+
+def test_sdpa_flux_full_size_sampled(dthip, oracle, torch_cuda):
+    """BASELINE shape (1, 24 heads x 128, 512 text + 4096 image tokens): sampled rows of two heads against
+    the oracle, and the constant-V property over the whole output."""
+    torch = torch_cuda
+    rng = np.random.default_rng(9)
+    B, T, HW, H, D = 1, 512, 4096, 24, 128
+    S = T + HW
+    q, k, v = rand_qkv(rng, B, S, S, H, H, D)
+    scale = 1 / np.sqrt(D)
+    qd, kd, vd = (to_dev(torch, t) for t in (q, k, v))
+    print("sdpa full size", flush=True)
+    got = dthip.sdpa_segments([qd[:, :T], qd[:, T:]], [kd[:, :T], kd[:, T:]], [vd[:, :T], vd[:, T:]], scale).cpu().numpy()
+    rows = np.sort(rng.choice(S, size=48, replace=False))
+    rows[0], rows[-1] = 0, S - 1
+    for h in (0, 23):
+        want = oracle.C.sdpa(np.ascontiguousarray(q[:, rows, h:h + 1]), np.ascontiguousarray(k[:, :, h:h + 1]),
+                             np.ascontiguousarray(v[:, :, h:h + 1]), scale)
+        mx, rr = oracle.err_stats(got[:, rows, h:h + 1], want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (h, mx, rr)
+    vc = torch.from_numpy(f16(rng.standard_normal((1, 1, H, D)))).cuda().expand(B, S, H, D).contiguous()
+    oc = dthip.ScaledDotProductAttention(scale=scale)(qd, kd, vc)
+    assert float((oc.float() - vc.float()).abs().max()) <= 2e-3

@@ -1,0 +1,200 @@
+"""GPU parity: palettized Dense (K0 depalettize, K1 GEMM) against the CPU oracle, through the C ABI.
+
+Bars: palette lookup / index unpack bit-exact; GEMM outputs max-abs <= 2e-2 and rel-RMS <= 1e-3
+(fp16 outputs, fp32 accumulation on both sides)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, REL_RMS = 2e-2, 1e-3
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+
+    assert torch.cuda.is_available()
+    return torch
+
+
+def to_dev(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def make_weight(dthip, oracle, rng, N, K, q, nib, std=0.02):
+    packed, pal, idx = oracle.synth_qx_weight(rng, N, K, q, nib, std)
+    return dthip.QxTensor.from_packed(packed, q, nib, (N, K)), packed
+
+
+@pytest.mark.parametrize("q", [4, 5, 6, 7, 8])
+@pytest.mark.parametrize("nib", [32, 512, 4096, 24])
+def test_depalettize_bit_exact(dthip, oracle, torch_cuda, q, nib):
+    torch = torch_cuda
+    rng = np.random.default_rng(q * 1000 + nib)
+    for count in (1, 31, 32, 33, nib - 1, nib, nib + 1, 5 * nib + 77, 64 * 1024 + 8):
+        print("depalettize", q, nib, count, flush=True)
+        packed, pal, idx = oracle.synth_qx_weight(rng, 1, count, q, nib, 1.0)
+        w = dthip.QxTensor.from_packed(packed, q, nib, (1, count))
+        got = w.dequantize().cpu().numpy().reshape(-1)
+        want = oracle.C.depalettize(q, nib, count, packed)
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+CASES = [
+    # (M, N, K, q, nib)  -- chosen to hit: every palette placement, ragged M / N edges, both tile shapes
+    (256, 256, 256, 8, 16384),    # shared palettes, nib > K
+    (300, 200, 512, 6, 4096),     # shared palettes, ragged M and N (small tile)
+    (1100, 520, 512, 6, 4096),    # big tile, ragged M and N
+    (1024, 512, 1024, 4, 512),    # per-row palettes (nib < K, K % nib == 0)
+    (1024, 256, 2048, 5, 1024),   # per-row palettes
+    (128, 384, 768, 4, 512),      # nib < K, K % nib != 0 -> lookups from global memory
+    (257, 129, 320, 6, 4096),     # SD1.5-like K = 320
+    (64, 96, 96, 7, 64),          # small everything
+    (1024, 256, 512, 8, 512),     # q8 with nib == K (many palettes -> global or shared)
+    (130, 70, 100, 6, 32),        # K % 32 != 0 -> generic kernel
+    (130, 70, 128, 6, 24),        # nib % 32 != 0 -> generic kernel
+]
+
+
+@pytest.mark.parametrize("M,N,K,q,nib", CASES)
+def test_dense_qx_vs_oracle(dthip, oracle, torch_cuda, M, N, K, q, nib):
+    torch = torch_cuda
+    rng = np.random.default_rng(hash((M, N, K, q, nib)) % (2 ** 32))
+    print("dense", M, N, K, q, nib, flush=True)
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    w, packed = make_weight(dthip, oracle, rng, N, K, q, nib)
+    bias = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    d = dthip.Dense(count=N, name="x_q")
+    d.weight, d.bias = w, to_dev(torch, bias)
+    got = d(to_dev(torch, X)).cpu().numpy()
+    want = oracle.C.dense_qx(X, packed, q, nib, N, bias)
+    mx, rr = oracle.err_stats(got, want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+    # no-bias variant
+    d2 = dthip.Dense(count=N, noBias=True)
+    d2.weight = w
+    got2 = d2(to_dev(torch, X)).cpu().numpy()
+    mx, rr = oracle.err_stats(got2, oracle.C.dense_qx(X, packed, q, nib, N, None))
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+@pytest.mark.parametrize("q,nib,K,N", [(8, 16384, 256, 320), (6, 4096, 512, 256), (5, 1024, 2048, 256),
+                                       (4, 512, 1024, 300), (4, 512, 768, 128), (7, 8192, 128, 256)])
+def test_effective_weights_bit_exact(dthip, oracle, torch_cuda, q, nib, K, N):
+    """X = I_K makes Y = W^T exactly (one nonzero product per output, fp16-representable):
+    the weights the fused kernel multiplies by are bit-for-bit the dequantized tensor."""
+    torch = torch_cuda
+    rng = np.random.default_rng(q + K)
+    print("effective weights", q, nib, K, N, flush=True)
+    w, packed = make_weight(dthip, oracle, rng, N, K, q, nib, std=1.0)
+    d = dthip.Dense(count=N, noBias=True)
+    d.weight = w
+    Y = d(to_dev(torch, np.eye(K, dtype=np.float16))).cpu().numpy()
+    W = oracle.C.depalettize(q, nib, N * K, packed).reshape(N, K)
+    assert np.array_equal(Y.view(np.uint16), np.ascontiguousarray(W.T).view(np.uint16))
+
+
+def test_dense_shared_input_three_weights_and_views(dthip, oracle, torch_cuda):
+    """x_q / x_k / x_v in one launch, input a strided row view, outputs written into one wide buffer."""
+    torch = torch_cuda
+    rng = np.random.default_rng(11)
+    M, K, N = 640, 512, 256
+    big = rng.standard_normal((M, K + 64)).astype(np.float16)
+    xb = to_dev(torch, big)
+    xv = xb[:, 32:32 + K]  # row stride K + 64, base offset 32 elements (16-byte aligned)
+    ws, packs, biases = [], [], []
+    for i in range(3):
+        w, p = make_weight(dthip, oracle, rng, N, K, 6, 4096)
+        ws.append(w)
+        packs.append(p)
+        biases.append((rng.standard_normal(N) * 0.02).astype(np.float16))
+    out = torch.zeros((M, 3 * N), dtype=torch.float16, device="cuda")
+    outs = [out[:, i * N:(i + 1) * N] for i in range(3)]
+    print("dense 3 weights", flush=True)
+    dthip.dense_multi(xv, ws, [to_dev(torch, b) for b in biases[:2]] + [None], outs=outs)
+    got = out.cpu().numpy()
+    X = np.ascontiguousarray(big[:, 32:32 + K])
+    for i in range(3):
+        want = oracle.C.dense_qx(X, packs[i], 6, 4096, N, biases[i] if i < 2 else None)
+        mx, rr = oracle.err_stats(got[:, i * N:(i + 1) * N], want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (i, mx, rr)
+
+
+def test_dense_plain_fp16_weight(dthip, oracle, torch_cuda):
+    torch = torch_cuda
+    rng = np.random.default_rng(12)
+    M, N, K = 333, 320, 320
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    W = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    b = (rng.standard_normal(N) * 0.05).astype(np.float16)
+    d = dthip.Dense(count=N)
+    d.weight, d.bias = dthip.QxTensor.from_f16(W), to_dev(torch, b)
+    print("dense fp16", flush=True)
+    got = d(to_dev(torch, X)).cpu().numpy()
+    mx, rr = oracle.err_stats(got, oracle.C.dense(X, W, b))
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+def test_dense_special_cases(dthip, oracle, torch_cuda):
+    torch = torch_cuda
+    rng = np.random.default_rng(13)
+    M, N, K, q, nib = 256, 256, 512, 6, 4096
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    nblocks = (N * K + nib - 1) // nib
+    idx = rng.integers(0, 1 << q, size=N * K, dtype=np.uint8)
+    b = rng.standard_normal(N).astype(np.float16)
+    # zero palette -> Y == bias exactly
+    w = dthip.QxTensor.from_packed(dthip.pack_qx(q, nib, np.zeros((nblocks, 1 << q), np.float16), idx), q, nib, (N, K))
+    d = dthip.Dense(count=N)
+    d.weight, d.bias = w, to_dev(torch, b)
+    print("dense special", flush=True)
+    assert np.array_equal(d(to_dev(torch, X)).cpu().numpy(), np.broadcast_to(b, (M, N)))
+    # single-valued palette -> Y = c * rowsum(X)
+    w = dthip.QxTensor.from_packed(dthip.pack_qx(q, nib, np.full((nblocks, 1 << q), 0.5, np.float16), idx), q, nib, (N, K))
+    d = dthip.Dense(count=N, noBias=True)
+    d.weight = w
+    got = d(to_dev(torch, X)).cpu().numpy().astype(np.float64)
+    want = 0.5 * X.astype(np.float64).sum(axis=1, keepdims=True) * np.ones((1, N))
+    assert np.max(np.abs(got - want)) <= np.max(np.abs(want)) * 2.0 ** -10 + 1e-3
+    # empty batch is a no-op
+    assert dthip.Dense.__call__(d, torch.zeros((0, K), dtype=torch.float16, device="cuda")).shape == (0, N)
+
+
+def test_dense_rejects_bad_arguments(dthip, torch_cuda):
+    torch = torch_cuda
+    w = dthip.QxTensor(torch.zeros(1024, dtype=torch.uint8, device="cuda"), 3, 32, (4, 32))
+    d = dthip.Dense(count=4, noBias=True)
+    d.weight = w
+    with pytest.raises(dthip.DtError) as e:
+        d(torch.zeros((8, 32), dtype=torch.float16, device="cuda"))
+    assert e.value.status == dthip.DT_INVALID
+
+
+def test_dense_flux_qkv_full_size_sampled(dthip, oracle, torch_cuda):
+    """BASELINE shape (M 4608, K 3072, three N 3072 q6p weights in one launch): a sample of rows
+    against the oracle, plus linearity Y(2x) == 2 Y(x) exactly (power-of-two scaling is exact in fp16/fp32)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(14)
+    M, K, N, q, nib = 4608, 3072, 3072, 6, 4096
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    ws, packs, biases = [], [], []
+    for i in range(3):
+        w, p = make_weight(dthip, oracle, rng, N, K, q, nib)
+        ws.append(w)
+        packs.append(p)
+        biases.append((rng.standard_normal(N) * 0.02).astype(np.float16))
+    xd = to_dev(torch, X)
+    print("dense full size", flush=True)
+    outs = dthip.dense_multi(xd, ws, [to_dev(torch, b) for b in biases])
+    rows = np.sort(rng.choice(M, size=24, replace=False))
+    rows[0], rows[-1] = 0, M - 1
+    for i in range(3):
+        got = outs[i].cpu().numpy()[rows]
+        want = oracle.C.dense_qx(np.ascontiguousarray(X[rows]), packs[i], q, nib, N, biases[i])
+        mx, rr = oracle.err_stats(got, want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (i, mx, rr)
+    o1 = dthip.dense_multi(xd, ws, [None] * 3)
+    o2 = dthip.dense_multi(xd * 2, ws, [None] * 3)
+    for a, b in zip(o1, o2):
+        assert torch.equal(a * 2, b)

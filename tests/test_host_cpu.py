@@ -1,0 +1,80 @@
+"""CPU-side checks of the product's host logic and of the C-ABI library as a binary:
+it loads, exports every declared symbol, and its pure-host entry points answer.
+No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(dthip):
+    header = open(os.path.join(ROOT, "include", "dt_hip.h")).read()
+    declared = set(re.findall(r"\b(dt_[a-z0-9_]+)\s*\(", header))
+    declared -= {"dt_status", "dt_stream"}
+    assert declared == set(dthip.ABI_SYMBOLS), declared ^ set(dthip.ABI_SYMBOLS)
+    L = ctypes.CDLL(dthip.LIB_PATH)
+    for name in declared:
+        assert hasattr(L, name), name
+
+
+def test_host_only_entry_points(dthip, oracle):
+    L = dthip.lib()
+    assert b"gfx950" in L.dt_version()
+    for q, nib in [(4, 512), (5, 1024), (6, 4096), (7, 64), (8, 16384)]:
+        for count in (0, 1, nib - 1, nib, 5 * nib + 3, 3072 * 3072):
+            assert dthip.qx_bytes(q, nib, count) == oracle.C.qx_bytes(q, nib, count)
+    assert dthip.qx_bytes(3, 32, 10) == -1 and dthip.qx_bytes(9, 32, 10) == -1 and dthip.qx_bytes(6, 0, 10) == -1
+    # workspace sizing: nothing needed for the plain call, Q'+K' for the fused prep, O for the fused projection
+    assert L.dt_sdpa_workspace_bytes(1, 24, 24, 128, 4608, 4608, 0, 0) == 0
+    one = 4608 * 24 * 128 * 2
+    assert L.dt_sdpa_workspace_bytes(1, 24, 24, 128, 4608, 4608, 1, 0) == 2 * one
+    assert L.dt_sdpa_workspace_bytes(1, 24, 24, 128, 4608, 4608, 1, 1) == 3 * one
+
+
+def test_missing_library_fails_loudly(dthip, monkeypatch):
+    monkeypatch.setattr(dthip, "_lib", None)
+    monkeypatch.setattr(dthip, "LIB_PATH", os.path.join(ROOT, "no_such_dir", "libdthip.so"))
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        dthip.lib()
+
+
+@pytest.mark.parametrize("q", [4, 5, 6, 7, 8])
+def test_host_packer_matches_oracle(dthip, oracle, q):
+    rng = np.random.default_rng(q)
+    for n in (0, 1, 7, 8, 9, 31, 32, 33, 1000):
+        idx = rng.integers(0, 1 << q, size=n, dtype=np.uint8)
+        assert np.array_equal(dthip.pack_indices(q, idx), oracle.C.pack_indices(q, idx))
+    for nib, count in [(32, 0), (32, 31), (32, 96), (64, 64 * 3 + 5), (512, 512 * 4)]:
+        nblocks = (count + nib - 1) // nib
+        pal = (rng.standard_normal((nblocks, 1 << q)) * 0.02).astype(np.float16)
+        idx = rng.integers(0, 1 << q, size=count, dtype=np.uint8)
+        assert np.array_equal(dthip.pack_qx(q, nib, pal, idx), oracle.C.palettize_pack(q, nib, pal, idx))
+
+
+def test_rotary_tables_match_oracle(dthip, oracle):
+    a = dthip.Flux1RotaryPositionEmbedding(6, 5, 4, channels=128)
+    assert np.array_equal(a, oracle.C.rope_flux(6, 5, 4, 128))
+    a = dthip.Flux1RotaryPositionEmbedding(4, 4, 2, referenceSizes=[(2, 3), (3, 2), (5, 1)], channels=128)
+    assert np.array_equal(a, oracle.C.rope_flux(4, 4, 2, 128, ref_sizes=[(2, 3), (3, 2), (5, 1)]))
+    a = dthip.Flux1RotaryPositionEmbedding(3, 7, 0, channels=64)
+    assert np.array_equal(a, oracle.C.rope_flux(3, 7, 0, 64))
+    w = dthip.WanRotaryPositionEmbedding(4, 5, 3, channels=128)
+    assert np.array_equal(w, oracle.C.rope_wan(4, 5, 3, 128))
+
+
+def test_instruction_counts(dthip, oracle):
+    assert dthip.DenseInstructionCount(4608, 3072, 9216) == oracle.C.dense_instruction_count(4608, 3072, 9216)
+    assert dthip.ScaledDotProductAttentionInstructionCount(1, 24, 128, 4608, 4608) == \
+        oracle.C.sdpa_instruction_count(1, 24, 128, 4608, 4608)
+
+
+def test_operator_surface_argument_checks(dthip):
+    with pytest.raises(dthip.DtError):
+        dthip.ScaledDotProductAttention(scale=1.0, isCausal=True)
+    d = dthip.Dense(count=8, noBias=True, name="x_q")
+    with pytest.raises(RuntimeError, match="weight not loaded"):
+        d(None)
