@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the transformer-block hot path on one MI355X.
+
+A "step" is one pass of the Flux.1-dev-shape double-stream joint attention block's hot path
+(512 text + 4096 image tokens, 24 heads x 128, q6p weights): two fused-QKV palettized Dense launches
+(text M=512, image M=4096; three 3072->3072 weights each), the QK RMSNorm + RoPE pass, joint
+ScaledDotProductAttention over 4608 tokens, and the two palettized output projections.
+All inputs are resident in HBM before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--kernel-iters", type=int, default=20, help="launches per kernel for the per-kernel timings")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    pkg = importlib.import_module("draw-things-community_amd")
+    L = pkg.lib()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    assert L.dt_init(0) == 0, "device 0 is not gfx950"
+    dev = torch.device("cuda:0")
+
+    # ---------------- workload: Flux joint block, q6p -----------------
+    T, HW, H, D = 512, 4096, 24, 128
+    S, C = T + HW, H * D
+    qbits, nib = pkg.CODEC["q6p"]
+    rng = np.random.default_rng(0)
+
+    def synth_weight():
+        count = C * C
+        nblocks = (count + nib - 1) // nib
+        pal = (rng.standard_normal((nblocks, 1 << qbits)) * 0.02).astype(np.float16)
+        idx = rng.integers(0, 1 << qbits, size=count, dtype=np.uint8)
+        packed = pkg.pack_qx(qbits, nib, pal, idx)
+        return pkg.QxTensor.from_packed(packed, qbits, nib, (C, C)), packed
+
+    def f16(shape, std=1.0):
+        return torch.from_numpy((rng.standard_normal(shape) * std).astype(np.float16)).to(dev)
+
+    w, packed_host, bias = {}, {}, {}
+    for name in ("c_q", "c_k", "c_v", "x_q", "x_k", "x_v", "c_o", "x_o"):
+        w[name], packed_host[name] = synth_weight()
+        bias[name] = f16((C,), 0.02)
+    gamma = {n: (1 + 0.02 * torch.randn(D, device=dev)).half() for n in ("c_q", "c_k", "x_q", "x_k")}
+    rot = torch.from_numpy(pkg.Flux1RotaryPositionEmbedding(64, 64, T, channels=D).astype(np.float16)).to(dev)
+    ctx = f16((T, C))
+    img = f16((HW, C))
+    # fused QKV outputs land in one [S, 3, H, D] buffer: text rows first, then image rows
+    qkv = torch.empty((S, 3, H, D), dtype=torch.float16, device=dev)
+    att = torch.empty((1, S, H, D), dtype=torch.float16, device=dev)
+    out_c = torch.empty((T, C), dtype=torch.float16, device=dev)
+    out_x = torch.empty((HW, C), dtype=torch.float16, device=dev)
+    scale = 1.0 / float(np.sqrt(D))
+    qkv2 = qkv.view(S, 3 * C)
+    views = lambda lo, hi: [qkv2[lo:hi, i * C:(i + 1) * C] for i in range(3)]
+    q4 = qkv[:, 0].unsqueeze(0)
+    k4 = qkv[:, 1].unsqueeze(0)
+    v4 = qkv[:, 2].unsqueeze(0)
+    att2 = att.view(S, C)
+
+    def k_qkv_text():
+        pkg.dense_multi(ctx, [w["c_q"], w["c_k"], w["c_v"]], [bias["c_q"], bias["c_k"], bias["c_v"]], outs=views(0, T))
+
+    def k_qkv_image():
+        pkg.dense_multi(img, [w["x_q"], w["x_k"], w["x_v"]], [bias["x_q"], bias["x_k"], bias["x_v"]], outs=views(T, S))
+
+    def k_prep():
+        for t4, gc, gx in ((q4, gamma["c_q"], gamma["x_q"]), (k4, gamma["c_k"], gamma["x_k"])):
+            pkg.qk_norm_rope_(t4[:, :T], gc, 1e-6, True, rot=rot, rot_pos0=0)
+            pkg.qk_norm_rope_(t4[:, T:], gx, 1e-6, True, rot=rot, rot_pos0=T)
+
+    def k_sdpa():
+        pkg.sdpa_segments([q4], [k4], [v4], scale, out=att)
+
+    def k_out():
+        pkg.dense_multi(att2[:T], [w["c_o"]], [bias["c_o"]], outs=[out_c])
+        pkg.dense_multi(att2[T:], [w["x_o"]], [bias["x_o"]], outs=[out_x])
+
+    def step():
+        k_qkv_text()
+        k_qkv_image()
+        k_prep()
+        k_sdpa()
+        k_out()
+
+    flop_dense = 2.0 * S * C * C * 4          # 6 QKV + 2 out projections, per-stream rows
+    flop_sdpa = 4.0 * H * S * S * D
+    flop_block = flop_dense + flop_sdpa
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / max(args.steps, 1)
+    value = flop_block / (ms_per_step * 1e-3) / 1e12
+
+    # ---------------- per-kernel timings (events on the launch stream) ----------------
+    def time_kernel(fn, iters):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    it = args.kernel_iters
+    ms = {
+        "dense_qkv_image_M4096": time_kernel(k_qkv_image, it),
+        "dense_qkv_text_M512": time_kernel(k_qkv_text, it),
+        "qk_norm_rope": time_kernel(k_prep, it),
+        "sdpa_S4608": time_kernel(k_sdpa, it),
+        "dense_out_2x": time_kernel(k_out, it),
+    }
+    # BASELINE "palettized Dense alone" shape: M = 4608, 3072 -> 9216 (three weights) and 3072 -> 3072
+    x_all = f16((S, C))
+    y3 = [torch.empty((S, C), dtype=torch.float16, device=dev) for _ in range(3)]
+    ms["dense_qkv_M4608_N9216"] = time_kernel(
+        lambda: pkg.dense_multi(x_all, [w["x_q"], w["x_k"], w["x_v"]], [bias["x_q"], bias["x_k"], bias["x_v"]], outs=y3), it)
+    ms["dense_out_M4608_N3072"] = time_kernel(
+        lambda: pkg.dense_multi(x_all, [w["x_o"]], [bias["x_o"]], outs=[y3[0]]), it)
+    wf16 = pkg.QxTensor.from_f16(w["x_q"].dequantize())
+    ms["dense_plainf16_M4608_N3072"] = time_kernel(
+        lambda: pkg.dense_multi(x_all, [wf16], [bias["x_o"]], outs=[y3[0]]), it)
+
+    tf = lambda flop, t_ms: flop / (t_ms * 1e-3) / 1e12
+    kernels = {
+        "sdpa_S4608": {"ms": ms["sdpa_S4608"], "tflops": tf(flop_sdpa, ms["sdpa_S4608"]),
+                       "ref_units_G": pkg.ScaledDotProductAttentionInstructionCount(1, H, D, S, S) / 1e9},
+        "dense_qkv_M4608_N9216_q6p": {"ms": ms["dense_qkv_M4608_N9216"], "tflops": tf(2.0 * S * C * 3 * C, ms["dense_qkv_M4608_N9216"])},
+        "dense_out_M4608_N3072_q6p": {"ms": ms["dense_out_M4608_N3072"], "tflops": tf(2.0 * S * C * C, ms["dense_out_M4608_N3072"])},
+        "dense_plainf16_M4608_N3072": {"ms": ms["dense_plainf16_M4608_N3072"], "tflops": tf(2.0 * S * C * C, ms["dense_plainf16_M4608_N3072"])},
+        "dense_qkv_image_M4096": {"ms": ms["dense_qkv_image_M4096"], "tflops": tf(2.0 * HW * C * 3 * C, ms["dense_qkv_image_M4096"])},
+        "dense_qkv_text_M512": {"ms": ms["dense_qkv_text_M512"], "tflops": tf(2.0 * T * C * 3 * C, ms["dense_qkv_text_M512"])},
+        "dense_out_2x": {"ms": ms["dense_out_2x"], "tflops": tf(2.0 * S * C * C, ms["dense_out_2x"])},
+        "qk_norm_rope": {"ms": ms["qk_norm_rope"], "gbs": 2 * 2 * S * C * 2 / (ms["qk_norm_rope"] * 1e-3) / 1e9},
+    }
+    for k in kernels.values():
+        if "tflops" in k:
+            k["frac_f16_peak"] = k["tflops"] / PEAK_F16_TFLOPS
+        k["ms"] = round(k["ms"], 4)
+
+    # dominant kernel of the step (by time): roofline against the fp16 MFMA peak
+    dense_ms = ms["dense_qkv_image_M4096"] + ms["dense_qkv_text_M512"] + ms["dense_out_2x"]
+    if ms["sdpa_S4608"] >= ms["dense_qkv_image_M4096"]:
+        dom, dom_flop, dom_ms = "sdpa_kernel<128,2> S=4608 H=24", flop_sdpa, ms["sdpa_S4608"]
+    else:
+        dom, dom_flop, dom_ms = "dense_qx_kernel<6,256,256> M=4096 N=3x3072 K=3072", 2.0 * HW * C * 3 * C, ms["dense_qkv_image_M4096"]
+    roofline = {
+        "kernel": dom, "bound": "mfma", "achieved": round(tf(dom_flop, dom_ms), 2), "peak": PEAK_F16_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(tf(dom_flop, dom_ms) / PEAK_F16_TFLOPS, 4), "traffic": None,
+        "flop_per_launch": dom_flop, "avg_launch_ms": round(dom_ms, 4),
+    }
+
+    # ---------------- CPU baseline: the oracle on a bounded sample ----------------
+    cpu = None
+    if not args.no_cpu:
+        from oracle import oracle
+
+        oracle.build()
+        ncores = oracle.C.lib.dto_num_threads()
+        m_s, rows_s, heads_s = 192, 768, 2
+        xs = (rng.standard_normal((m_s, C))).astype(np.float16)
+        t0 = time.perf_counter()
+        for name in ("x_q", "x_k", "x_v", "x_o"):
+            oracle.C.dense_qx(xs, packed_host[name], qbits, nib, C, None)
+        t_dense = time.perf_counter() - t0
+        qs = rng.standard_normal((1, rows_s, heads_s, D)).astype(np.float16)
+        ks = rng.standard_normal((1, S, heads_s, D)).astype(np.float16)
+        vs = rng.standard_normal((1, S, heads_s, D)).astype(np.float16)
+        t0 = time.perf_counter()
+        oracle.C.sdpa(qs, ks, vs, scale)
+        t_sdpa = time.perf_counter() - t0
+        f_dense = 2.0 * m_s * C * C * 4
+        f_sdpa = 4.0 * heads_s * rows_s * S * D
+        # time for the whole block at the sample's rates, then block FLOPs over it
+        t_block = t_dense * (flop_dense / f_dense) + t_sdpa * (flop_sdpa / f_sdpa)
+        cpu = {
+            "value": round(flop_block / t_block / 1e12, 5), "unit": "TFLOP/s", "cores": int(ncores), "kind": "port",
+            "sample": f"oracle (C, OpenMP): 4 q6p Dense 3072->3072 on {m_s} rows ({t_dense:.2f} s, depalettize included) + "
+                      f"attention of {rows_s} query rows x {heads_s} heads against all {S} keys ({t_sdpa:.2f} s); "
+                      "block time extrapolated linearly in rows/heads",
+            "dense_gflops": round(f_dense / t_dense / 1e9, 1), "sdpa_gflops": round(f_sdpa / t_sdpa / 1e9, 1),
+        }
+
+    line = {
+        "metric": "SDPA + palettized-GEMM TFLOP/s (% fp16 peak); ms/block, Flux 4608 tok q6p",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "Flux.1-dev joint attention block hot path: 512 text + 4096 image tokens, 24x128 heads, "
+                               "q6p (nib 4096) weights; 6 QKV Dense + QK RMSNorm/RoPE + SDPA + 2 out-proj Dense",
+                   "flop_per_block": flop_block, "frac_f16_peak": round(value / PEAK_F16_TFLOPS, 4)},
+        "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels,
+        "block_ms_sum_of_kernels": round(dense_ms + ms["sdpa_S4608"] + ms["qk_norm_rope"], 4),
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -384,7 +384,7 @@ DT_EXPORT dt_status dt_dense_qx_f16(dt_stream stream, int64_t M, int64_t K, cons
     if (!w.data || w.count < 0 || w.count % K != 0) return DT_INVALID;
     if (w.qbits != 16 && (w.qbits < 4 || w.qbits > 8 || w.nib <= 0)) return DT_INVALID;
     if (w.count / K > 0x7fffffff) return DT_INVALID;
-    if (!Y[i] || ldy[i] < w.count / K) return DT_INVALID;
+    if (M > 0 && (!Y[i] || ldy[i] < w.count / K)) return DT_INVALID;
   }
   if (M == 0) return DT_OK;
   if (!X || ldx < K) return DT_INVALID;

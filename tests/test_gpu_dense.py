@@ -173,7 +173,7 @@ def test_dense_rejects_bad_arguments(dthip, torch_cuda):
 
 def test_dense_flux_qkv_full_size_sampled(dthip, oracle, torch_cuda):
     """BASELINE shape (M 4608, K 3072, three N 3072 q6p weights in one launch): a sample of rows
-    against the oracle, plus linearity Y(2x) == 2 Y(x) exactly (power-of-two scaling is exact in fp16/fp32)."""
+    against the oracle, plus linearity Y(2x) == 2 Y(x) (power-of-two scaling is exact in fp32 and in normal fp16)."""
     torch = torch_cuda
     rng = np.random.default_rng(14)
     M, K, N, q, nib = 4608, 3072, 3072, 6, 4096
@@ -197,4 +197,7 @@ def test_dense_flux_qkv_full_size_sampled(dthip, oracle, torch_cuda):
     o1 = dthip.dense_multi(xd, ws, [None] * 3)
     o2 = dthip.dense_multi(xd * 2, ws, [None] * 3)
     for a, b in zip(o1, o2):
-        assert torch.equal(a * 2, b)
+        # exact wherever 2y is a normal fp16 number; subnormal results may round differently
+        normal = a.abs() >= 2.0 ** -13
+        assert torch.equal((a * 2)[normal], b[normal])
+        assert float((a.float() * 2 - b.float()).abs().max()) <= 2.0 ** -23
