@@ -12,6 +12,7 @@
 // K-tile and the unpack VALU/LDS work overlaps the matrix pipe.
 #include "dt_common.h"
 #include "dt_layout.h"
+#include <cstdlib>
 
 namespace dt {
 
@@ -50,24 +51,58 @@ __device__ __forceinline__ uint4_t ld_global_16(const void* p) {
   return *reinterpret_cast<const uint4_t*>(p);
 }
 
-template <int Q, int BM, int BN, int MODE>
-__global__ void __launch_bounds__(256) dense_qx_kernel(const DenseArgs a) {
-  constexpr int WM = BM / 2, WN = BN / 2;  // per-wave output tile
-  constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int A_CHUNKS = BM * (BK / 8) / 256;  // 16-byte chunks of X per thread per K-tile
-  constexpr int B_GRAN = BN / 256 > 0 ? BN / 256 : 1;  // 32-index granules per thread per K-tile
-  constexpr int B_CHUNKS = BN * (BK / 8) / 256;        // plain fp16 weight: 16-byte chunks per thread
-  constexpr int QW = MODE == kPlainF16 ? 1 : Q;        // dwords per granule
-  static_assert(BM % 64 == 0 && BN % 64 == 0, "tile");
+// Per-thread cursor over one weight row's packed indices, advanced one K-tile
+// (32 elements) at a time so the main loop needs no division.
+struct RowCursor {
+  uint32_t off;   // byte offset of the current granule's first index dword
+  uint32_t poff;  // byte offset of the current block's palette
+  int32_t r;      // element offset inside the current block (multiple of 32)
+  int32_t slot;   // palette slot in LDS (shared mode: block - first block of the tile)
+};
 
-  __shared__ __attribute__((aligned(16))) half_t As[2][BM * LDS_ROW];
-  __shared__ __attribute__((aligned(16))) half_t Bs[2][BN * LDS_ROW];
+// LDS tiles are [rows][32 halfs] with 64-byte rows and no padding; the 16-byte
+// chunk c of row r lives at chunk c ^ ((r >> 2) & 3).  The LDS of this part
+// serves 16 lanes of a 16-byte access per clock over 64 banks, so 16
+// consecutive rows of one chunk column (the MFMA operand reads and the
+// unpackers' row-per-lane writes) must land on 16 distinct 16-byte bank
+// groups: 4 * (r % 4) + (c ^ (r / 4 % 4)) does.  Measured conflict-free for
+// the operand reads, the 4-lanes-per-row tile writes and the row-per-lane writes.
+__device__ __forceinline__ int lds_chunk(int row, int c) { return row * BK + ((c ^ ((row >> 2) & 3)) << 3); }
+
+__device__ __forceinline__ uint32_t pack_h2(float a, float b) {
+  return (uint32_t)half_to_bits((half_t)a) | ((uint32_t)half_to_bits((half_t)b) << 16);
+}
+
+// 512 threads = 8 waves, two per SIMD.  Every thread stages two 16-byte chunks
+// of the X tile and unpacks / looks up half a granule (16 weights) of one W
+// row per K-tile, so the LDS instructions -- which a single wave can only
+// issue every few tens of clocks -- are spread evenly over all eight waves.
+// Waves w and w+4 share a SIMD and run the two halves of an iteration in
+// opposite order, so one of them is always feeding the matrix pipe.  All
+// eight run MFMAs on a (BN/2) x (BM/4) slice.  The accumulators are held
+// transposed (rows = output features n, columns = tokens m) so that each lane
+// ends up with runs of consecutive n for one token: 16-byte stores.
+template <int Q, int BM, int BN, int MODE, int EXP = 0>
+__global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
+  constexpr int WN = BN / 2, WM = BM / 4;   // per-wave slice: WN features x WM tokens
+  constexpr int TN = WN / 32, TM = WM / 32;
+  constexpr int A_CHUNKS = BM * (BK / 8) / 512;  // 16-byte chunks of X per thread per K-tile
+  constexpr int B_CHUNKS = BN * (BK / 8) / 512;  // plain fp16 weight: 16-byte chunks per thread
+  constexpr int QW = MODE == kPlainF16 ? 1 : Q;  // dwords per granule
+  constexpr int NST = 3;                         // LDS ring depth
+  constexpr int A_STAGE = BM * BK, B_STAGE = BN * BK;
+  static_assert(BM % 128 == 0 && BN % 64 == 0 && BN <= 256, "tile");
+
+  __shared__ __attribute__((aligned(16))) half_t As[NST * A_STAGE];
+  __shared__ __attribute__((aligned(16))) half_t Bs[NST * B_STAGE];
   __shared__ __attribute__((aligned(16))) uint16_t Pal[(MODE == kPalShared || MODE == kPalRow) ? kPalLdsBytes / 2 : 8];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const bool second = wave >= 4;     // stages first, then runs its MFMAs; unpacks weights 16..31 of its granule
+  const int lt = tid & 255;
+  const int wn = wave & 1, wm = (wave >> 1) & 1 | ((wave >> 2) << 1);  // waves w and w+4 share a SIMD and take different m slices
 
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous
   // run of tiles so the weight tiles it re-reads stay in that XCD's L2.
@@ -88,57 +123,75 @@ __global__ void __launch_bounds__(256) dense_qx_kernel(const DenseArgs a) {
   const int n0 = (tn - w.tile_begin) * BN;
   const int m0 = tm * BM;
   const int K = a.k;
+  const int nk = K / BK;
   const QxLayout lay = make_layout(Q, a.nib);
+  const uint32_t pal_bytes = (uint32_t)lay.pal_bytes;
+  // Rows of X (and of a plain fp16 W) are K * 2 bytes apart, a stride that maps
+  // a K-tile's 64-byte row segments onto very few memory channels.  Each
+  // workgroup walks the K-tiles in a rotated order so that concurrent
+  // workgroups pull from different channels.
+  const int rot = (int)(((unsigned)tm * 5u + (unsigned)tn * 11u) % (unsigned)nk);
 
-  // ---- per-thread load coordinates -------------------------------------
-  const uint16_t* a_src[A_CHUNKS];
+  // ---- per-thread load coordinates (32-bit byte offsets from uniform bases) ----
+  uint32_t a_off[A_CHUNKS];
   int a_dst[A_CHUNKS];
 #pragma unroll
   for (int i = 0; i < A_CHUNKS; i++) {
-    int c = tid + i * 256;
+    int c = tid + i * 512;
     int row = c >> 2, kc = c & 3;
     int gm = m0 + row;
     if (gm >= a.m) gm = a.m - 1;
-    a_src[i] = a.x + (int64_t)gm * a.ldx + kc * 8;
-    a_dst[i] = row * LDS_ROW + kc * 8;
+    a_off[i] = (uint32_t)(((int64_t)gm * a.ldx + kc * 8) * 2);
+    a_dst[i] = lds_chunk(row, kc);
   }
-  // weight rows handled by this thread (palettized: one granule per row per K-tile)
-  int b_row[B_GRAN];
-  int64_t b_flat[B_GRAN];  // flat element index of (row, k = 0)
-#pragma unroll
-  for (int g = 0; g < B_GRAN; g++) {
-    int row = tid + g * 256;
-    b_row[g] = row;
-    int gn = n0 + row;
+  const char* xbase = reinterpret_cast<const char*>(a.x);
+  const char* wbase = reinterpret_cast<const char*>(w.data);
+
+  // weight row of this thread (both threads of a pair read the row's granule, each unpacks one half)
+  const bool b_active = (BN >= 256) || (lt < BN);
+  const int b_row = lt < BN ? lt : BN - 1;
+  RowCursor cur, cur0;  // current tile, and tile 0 for the wrap-around
+  int64_t pal_first_block = 0;
+  if constexpr (MODE == kPalShared) pal_first_block = ((int64_t)n0 * K) / a.nib;
+  if constexpr (MODE != kPlainF16) {
+    int gn = n0 + b_row;
     if (gn >= w.n) gn = w.n - 1;
-    b_flat[g] = (int64_t)gn * K;
+    auto cursor_at = [&](int tile) {
+      const int64_t e = (int64_t)gn * K + (int64_t)tile * BK;
+      const int64_t blk = e / a.nib;
+      const int64_t r = e - blk * a.nib;
+      RowCursor c;
+      c.off = (uint32_t)index_byte_offset(lay, blk, r);
+      c.poff = (uint32_t)palette_offset(lay, blk);
+      c.r = (int32_t)r;
+      c.slot = MODE == kPalShared ? (int32_t)(blk - pal_first_block) : b_row;
+      return c;
+    };
+    cur = cursor_at(rot);
+    cur0 = cursor_at(0);
   }
-  const bool b_active = (BN >= 256) || (tid < BN);
-  // plain fp16 weight: same chunking as X
-  const uint16_t* bf_src[B_CHUNKS];
-  int bf_dst[B_CHUNKS];
+  uint32_t bf_off[B_CHUNKS > 0 ? B_CHUNKS : 1];
+  int bf_dst[B_CHUNKS > 0 ? B_CHUNKS : 1];
   if constexpr (MODE == kPlainF16) {
 #pragma unroll
     for (int i = 0; i < B_CHUNKS; i++) {
-      int c = tid + i * 256;
+      int c = tid + i * 512;
       int row = c >> 2, kc = c & 3;
       int gn = n0 + row;
       if (gn >= w.n) gn = w.n - 1;
-      bf_src[i] = reinterpret_cast<const uint16_t*>(w.data) + (int64_t)gn * K + kc * 8;
-      bf_dst[i] = row * LDS_ROW + kc * 8;
+      bf_off[i] = (uint32_t)(((int64_t)gn * K + kc * 8) * 2);
+      bf_dst[i] = lds_chunk(row, kc);
     }
   }
 
   // ---- palettes -> LDS --------------------------------------------------
-  int64_t pal_first_block = 0;
   if constexpr (MODE == kPalShared) {
     int last_row = n0 + BN - 1;
     if (last_row >= w.n) last_row = w.n - 1;
-    pal_first_block = ((int64_t)n0 * K) / a.nib;
     int64_t last_block = ((int64_t)last_row * K + (K - 1)) / a.nib;
     int n_pal = (int)(last_block - pal_first_block + 1);
     const int per_pal = 1 << (Q - 1);  // dwords per palette
-    for (int i = tid; i < n_pal * per_pal; i += 256) {
+    for (int i = tid; i < n_pal * per_pal; i += 512) {
       int p = i / per_pal, e = i - p * per_pal;
       const uint32_t* src =
           reinterpret_cast<const uint32_t*>(w.data + palette_offset(lay, pal_first_block + p));
@@ -149,7 +202,7 @@ __global__ void __launch_bounds__(256) dense_qx_kernel(const DenseArgs a) {
     // kPalRow: block of row n at column k0 is n * (K / nib) + k0 / nib
     const int per_pal = 1 << (Q - 1);
     const int bpr = K / a.nib;
-    for (int i = tid; i < BN * per_pal; i += 256) {
+    for (int i = tid; i < BN * per_pal; i += 512) {
       int row = i / per_pal, e = i - row * per_pal;
       int gn = n0 + row;
       if (gn >= w.n) gn = w.n - 1;
@@ -158,139 +211,244 @@ __global__ void __launch_bounds__(256) dense_qx_kernel(const DenseArgs a) {
       reinterpret_cast<uint32_t*>(Pal)[i] = src[e];
     }
   };
-  if constexpr (MODE == kPalRow) load_row_palettes(0);
+  if constexpr (MODE == kPalRow) load_row_palettes(rot * BK);
 
-  // ---- register staging -------------------------------------------------
-  uint4_t a_reg[A_CHUNKS];
-  uint32_t b_raw[B_GRAN][QW];
-  uint4_t bf_reg[B_CHUNKS];
+  // ---- register staging: two sets so a tile's loads fly for a whole iteration ----
+  struct RegSet {
+    uint4_t x[A_CHUNKS];
+    uint4_t wf[B_CHUNKS > 0 ? B_CHUNKS : 1];  // plain fp16 weight chunks
+    uint32_t b[QW];                           // packed indices of the row's granule
+    uint32_t poff;
+    int32_t slot;
+  };
+  RegSet R0, R1, R2;
 
-  auto issue_loads = [&](int k0) {
+  // Loads the tile the cursor points at (the last tile is re-read harmlessly by
+  // the final iterations) and moves the cursor on by one tile.
+  int next_tile = rot;  // K-tile the cursor points at
+  int issued = 0;       // tiles loaded so far
+  auto issue_loads = [&](RegSet& R) {
+    const int k0 = next_tile * BK;
+    const char* xk = xbase + (int64_t)k0 * 2;
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; i++) a_reg[i] = ld_global_16(a_src[i] + k0);
+    for (int i = 0; i < A_CHUNKS; i++) R.x[i] = ld_global_16(xk + a_off[i]);
     if constexpr (MODE == kPlainF16) {
+      const char* wk = wbase + (int64_t)k0 * 2;
 #pragma unroll
-      for (int i = 0; i < B_CHUNKS; i++) bf_reg[i] = ld_global_16(bf_src[i] + k0);
+      for (int i = 0; i < B_CHUNKS; i++) R.wf[i] = ld_global_16(wk + bf_off[i]);
     } else {
-      if (b_active) {
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(wbase + cur.off);
 #pragma unroll
-        for (int g = 0; g < B_GRAN; g++) {
-          int64_t e = b_flat[g] + k0;
-          int64_t blk = e / a.nib;
-          int64_t r = e - blk * a.nib;
-          const uint32_t* src = reinterpret_cast<const uint32_t*>(w.data + index_byte_offset(lay, blk, r));
-#pragma unroll
-          for (int i = 0; i < QW; i++) b_raw[g][i] = src[i];
+      for (int i = 0; i < QW; i++) R.b[i] = src[i];
+      R.poff = cur.poff;
+      R.slot = cur.slot;
+    }
+    if (issued + 1 < nk) {
+      issued++;
+      next_tile++;
+      if (next_tile == nk) {
+        next_tile = 0;
+        if constexpr (MODE != kPlainF16) cur = cur0;
+      } else if constexpr (MODE != kPlainF16) {
+        cur.r += BK;
+        cur.off += 4 * Q;
+        if (cur.r >= a.nib) {
+          cur.r = 0;
+          cur.off += pal_bytes;
+          cur.poff += (uint32_t)lay.block_stride;
+          if constexpr (MODE == kPalShared) cur.slot++;
         }
       }
     }
   };
 
-  auto stage_to_lds = [&](int stage, int k0) {
+  auto stage_to_lds = [&](const RegSet& R, int stage) {
+    half_t* Asd = As + stage * A_STAGE;
+    half_t* Bsd = Bs + stage * B_STAGE;
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; i++) *reinterpret_cast<uint4_t*>(&As[stage][a_dst[i]]) = a_reg[i];
+    for (int i = 0; i < A_CHUNKS; i++) *reinterpret_cast<uint4_t*>(&Asd[a_dst[i]]) = R.x[i];
     if constexpr (MODE == kPlainF16) {
 #pragma unroll
-      for (int i = 0; i < B_CHUNKS; i++) *reinterpret_cast<uint4_t*>(&Bs[stage][bf_dst[i]]) = bf_reg[i];
+      for (int i = 0; i < B_CHUNKS; i++) *reinterpret_cast<uint4_t*>(&Bsd[bf_dst[i]]) = R.wf[i];
     } else {
       if (b_active) {
+        uint32_t idx[16];
+        if (second)
+          unpack16<Q, 1>(R.b, idx);
+        else
+          unpack16<Q, 0>(R.b, idx);
+        uint32_t o[8];
+        const uint16_t* pal;
+        if constexpr (MODE == kPalGlobal)
+          pal = reinterpret_cast<const uint16_t*>(wbase + R.poff);
+        else
+          pal = Pal + (R.slot << Q);
 #pragma unroll
-        for (int g = 0; g < B_GRAN; g++) {
-          uint32_t idx[32];
-          unpack32<Q>(b_raw[g], idx);
-          uint32_t o[16];
-          if constexpr (MODE == kPalGlobal) {
-            int64_t blk = (b_flat[g] + k0) / a.nib;
-            const uint16_t* pal = reinterpret_cast<const uint16_t*>(w.data + palette_offset(lay, blk));
-#pragma unroll
-            for (int j = 0; j < 16; j++)
-              o[j] = (uint32_t)pal[idx[2 * j]] | ((uint32_t)pal[idx[2 * j + 1]] << 16);
-          } else {
-            int slot;
-            if constexpr (MODE == kPalShared)
-              slot = (int)((b_flat[g] + k0) / a.nib - pal_first_block);
-            else
-              slot = b_row[g];
-            const uint16_t* pal = Pal + (slot << Q);
-#pragma unroll
-            for (int j = 0; j < 16; j++)
-              o[j] = (uint32_t)pal[idx[2 * j]] | ((uint32_t)pal[idx[2 * j + 1]] << 16);
-          }
-          uint4_t* dst = reinterpret_cast<uint4_t*>(&Bs[stage][b_row[g] * LDS_ROW]);
-#pragma unroll
-          for (int j = 0; j < 4; j++) dst[j] = uint4_t{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
-        }
+        for (int j = 0; j < 8; j++) o[j] = (uint32_t)pal[idx[2 * j]] | ((uint32_t)pal[idx[2 * j + 1]] << 16);
+        const int c0 = second ? 2 : 0;
+        *reinterpret_cast<uint4_t*>(&Bsd[lds_chunk(b_row, c0)]) = uint4_t{o[0], o[1], o[2], o[3]};
+        *reinterpret_cast<uint4_t*>(&Bsd[lds_chunk(b_row, c0 + 1)]) = uint4_t{o[4], o[5], o[6], o[7]};
       }
     }
   };
 
-  float16_t acc[TM][TN];
+  float16_t acc[TN][TM];
 #pragma unroll
-  for (int i = 0; i < TM; i++)
+  for (int i = 0; i < TN; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+    for (int j = 0; j < TM; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-  const int nk = K / BK;
-  issue_loads(0);
-  __syncthreads();  // palettes visible
-  stage_to_lds(0, 0);
-  __syncthreads();
-
-  const int frag_row = lane & 31;
-  const int frag_k = (lane >> 5) * 8;
-
-  for (int kt = 0; kt < nk; kt++) {
-    const int cur = kt & 1;
-    const bool more = kt + 1 < nk;
-    if (more) issue_loads((kt + 1) * BK);
-
-    const half_t* Ab = &As[cur][(wm * WM + frag_row) * LDS_ROW + frag_k];
-    const half_t* Bb = &Bs[cur][(wn * WN + frag_row) * LDS_ROW + frag_k];
+  // ---- fragment double buffer --------------------------------------------
+  // MFMA A operand = W rows (features), B operand = X rows (tokens); lane holds
+  // row (lane & 31), k-slots 8 * (lane / 32) .. + 7 of the 16-wide k-step.
+  const int l32 = lane & 31, hi = lane >> 5;
+  half8_t fw[2][TN], fx[2][TM];
+  auto read_frags = [&](int buf, int stage, int ks) {
+    const half_t* Wb = Bs + stage * B_STAGE;
+    const half_t* Xb = As + stage * A_STAGE;
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ks++) {
-      half8_t af[TM], bf[TN];
+    for (int i = 0; i < TN; i++)
+      fw[buf][i] = *reinterpret_cast<const half8_t*>(Wb + lds_chunk(wn * WN + i * 32 + l32, 2 * ks + hi));
 #pragma unroll
-      for (int i = 0; i < TM; i++) af[i] = *reinterpret_cast<const half8_t*>(Ab + i * 32 * LDS_ROW + ks * 16);
+    for (int j = 0; j < TM; j++)
+      fx[buf][j] = *reinterpret_cast<const half8_t*>(Xb + lds_chunk(wm * WM + j * 32 + l32, 2 * ks + hi));
+  };
+  auto mfma_step = [&](int buf) {
 #pragma unroll
-      for (int j = 0; j < TN; j++) bf[j] = *reinterpret_cast<const half8_t*>(Bb + j * 32 * LDS_ROW + ks * 16);
+    for (int i = 0; i < TN; i++)
 #pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
-    }
-
-    if (more) {
-      const int k1 = (kt + 1) * BK;
-      if constexpr (MODE == kPalRow) {
-        if (k1 % a.nib == 0) {
-          // every lookup of the previous K-tile finished before the last barrier
-          load_row_palettes(k1);
-          __syncthreads();
+      for (int j = 0; j < TM; j++)
+        if constexpr (EXP & 32) {
+          asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fw[buf][i]), "v"(fx[buf][j]));
+        } else {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[buf][i], fx[buf][j], acc[i][j], 0, 0, 0);
         }
-      }
-      stage_to_lds(cur ^ 1, k1);
-    }
-    __syncthreads();
-  }
+  };
 
-  // ---- epilogue: bias, round once to fp16, store ------------------------
-  // accumulator layout of v_mfma_f32_32x32x16: lane holds column (lane & 31),
-  // rows 8 * (v / 4) + 4 * (lane / 32) + (v % 4).
+  // ---- prologue: tiles 0 and 1 into the ring, tiles 2 and 3 in flight ---------
+  issue_loads(R0);  // tile 0
+  issue_loads(R1);  // tile 1
+  issue_loads(R2);  // tile 2
+  __syncthreads();  // palettes visible
+  stage_to_lds(R0, 0);
+  issue_loads(R0);  // tile 3
+  if constexpr (MODE == kPalRow) {
+    const int k1 = ((rot + 1) % nk) * BK;
+    if (k1 % a.nib == 0 && nk > 1) {  // tile 1 already starts a new palette block
+      __syncthreads();
+      load_row_palettes(k1);
+      __syncthreads();
+    }
+  }
+  stage_to_lds(R1, 1);
+  __syncthreads();
+  read_frags(0, 0, 0);
+
+  // Iteration t: MFMAs of tile t from ring stage t % 3 while tile t+2 (loaded two
+  // iterations ago) is unpacked into stage (t+2) % 3 and tile t+4 starts loading.
+  // The fragments of the next k-step are always read one step ahead, across the
+  // barrier too (stage (t+1) % 3 was completed before the previous barrier).
+  // The two waves of a SIMD run the two halves of an iteration in opposite
+  // order (unpackers stage first, loaders run their MFMAs first), so one of
+  // them is always feeding the matrix pipe while the other does VALU / LDS work.
+  auto iteration = [&](int t, RegSet& Rstage, RegSet& Rload) {
+    const int s_cur = t % NST;
+    const int s_nxt = (t + 1) % NST;
+    const int s_fill = (t + 2) % NST;
+    if constexpr (!(EXP & 1)) issue_loads(Rload);
+    if constexpr (MODE == kPalRow) {
+      const int k2 = ((t + 2 + rot) % nk) * BK;
+      if (t + 2 < nk && k2 % a.nib == 0) {
+        // lookups of tile t+1 finished before the last barrier
+        load_row_palettes(k2);
+        __syncthreads();
+      }
+    }
+    if (second) {
+      if constexpr (!(EXP & 2)) stage_to_lds(Rstage, s_fill);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!(EXP & 8)) read_frags(1, s_cur, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!(EXP & 16)) mfma_step(0);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!(EXP & 8)) read_frags(0, s_nxt, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!(EXP & 16)) mfma_step(1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (!second) {
+      if constexpr (!(EXP & 2)) stage_to_lds(Rstage, s_fill);
+    }
+    if constexpr (!(EXP & 4)) __syncthreads();
+  };
+
+  // tile T travels in register set T % 3: iteration t stages set (t+2) % 3 and refills set (t+1) % 3
+  int t = 0;
+  for (; t + 2 < nk; t += 3) {
+    iteration(t, R2, R1);
+    iteration(t + 1, R0, R2);
+    iteration(t + 2, R1, R0);
+  }
+  if (t < nk) iteration(t, R2, R1);
+  if (t + 1 < nk) iteration(t + 1, R0, R2);
+
+  // ---- epilogue: bias, round once to fp16, 16-byte stores -------------------
+  // Accumulator block (i, j): lane holds token column (lane & 31) and features
+  // 8 * g + 4 * (lane / 32) + (0..3) for g = 0..3.  Swapping the odd groups of
+  // the low half-wave with the even groups of the high half-wave leaves every
+  // lane with runs of 8 consecutive features.
 #pragma unroll
-  for (int j = 0; j < TN; j++) {
-    const int gn = n0 + wn * WN + j * 32 + (lane & 31);
-    if (gn >= w.n) continue;
-    float bv = 0.f;
-    if (w.bias) bv = (float)bits_to_half(w.bias[gn]);
+  for (int j = 0; j < TM; j++) {
+    const int gm = m0 + wm * WM + j * 32 + l32;
+    uint16_t* yrow = w.y + (int64_t)(gm < a.m ? gm : 0) * w.ldy;
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
+    for (int i = 0; i < TN; i++) {
+      const int nb = n0 + wn * WN + i * 32;
+      uint32_t pk[4][2];
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const int gm = m0 + wm * WM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        if (gm < a.m) w.y[(int64_t)gm * w.ldy + gn] = half_to_bits((half_t)(acc[i][j][v] + bv));
+      for (int g = 0; g < 4; g++) {
+        float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+        if (w.bias) {
+          const int nn = nb + 8 * g + 4 * hi;
+          if (nn + 3 < w.n) {
+            const uint2_t bb = *reinterpret_cast<const uint2_t*>(w.bias + nn);
+            b0 = (float)bits_to_half((uint16_t)bb[0]);
+            b1 = (float)bits_to_half((uint16_t)(bb[0] >> 16));
+            b2 = (float)bits_to_half((uint16_t)bb[1]);
+            b3 = (float)bits_to_half((uint16_t)(bb[1] >> 16));
+          } else {
+            if (nn < w.n) b0 = (float)bits_to_half(w.bias[nn]);
+            if (nn + 1 < w.n) b1 = (float)bits_to_half(w.bias[nn + 1]);
+            if (nn + 2 < w.n) b2 = (float)bits_to_half(w.bias[nn + 2]);
+          }
+        }
+        pk[g][0] = pack_h2(acc[i][j][4 * g] + b0, acc[i][j][4 * g + 1] + b1);
+        pk[g][1] = pack_h2(acc[i][j][4 * g + 2] + b2, acc[i][j][4 * g + 3] + b3);
+      }
+      // after the swaps: low half-wave holds groups 0 and 2 complete (features
+      // 0..7, 16..23), high half-wave groups 1 and 3 (features 8..15, 24..31)
+#pragma unroll
+      for (int gp = 0; gp < 2; gp++) {
+        uint32_t run[4];
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+          // v_permlane32_swap: first operand's high half <-> second operand's low half
+          auto r = __builtin_amdgcn_permlane32_swap(pk[2 * gp][e], pk[2 * gp + 1][e], false, false);
+          run[e] = r[0];      // low lanes: own group 2gp     | high lanes: low lanes' group 2gp+1
+          run[2 + e] = r[1];  // low lanes: high lanes' 2gp   | high lanes: own group 2gp+1
+        }
+        const int nn = nb + 16 * gp + 8 * hi;
+        if (gm < a.m) {
+          if (nn + 7 < w.n && ((w.ldy & 7) == 0) && ((reinterpret_cast<uintptr_t>(w.y) & 15) == 0)) {
+            *reinterpret_cast<uint4_t*>(yrow + nn) = uint4_t{run[0], run[1], run[2], run[3]};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              if (nn + e < w.n) yrow[nn + e] = (uint16_t)(run[e >> 1] >> (16 * (e & 1)));
+          }
+        }
       }
     }
   }
@@ -328,7 +486,7 @@ __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* _
 
 template <int Q, int BM, int BN>
 static dt_status launch_tiled(hipStream_t s, const DenseArgs& a, int mode) {
-  dim3 grid((unsigned)(a.tiles_m * a.tiles_n)), block(256);
+  dim3 grid((unsigned)(a.tiles_m * a.tiles_n)), block(512);
   switch (mode) {
     case kPalShared: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalShared>), grid, block, 0, s, a); break;
     case kPalRow:
@@ -352,7 +510,24 @@ static dt_status launch_tiled_q(hipStream_t s, const DenseArgs& a, int qbits, in
     case 7: return launch_tiled<7, BM, BN>(s, a, mode);
     case 8: return launch_tiled<8, BM, BN>(s, a, mode);
     case 16: {
-      dim3 grid((unsigned)(a.tiles_m * a.tiles_n)), block(256);
+      dim3 grid((unsigned)(a.tiles_m * a.tiles_n)), block(512);
+      const char* ex = getenv("DT_DENSE_EXP");
+      int e = ex ? atoi(ex) : 0;
+      if constexpr (BM == 256) {
+        switch (e) {
+          case 1: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 1>), grid, block, 0, s, a); return launch_status();
+          case 2: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 2>), grid, block, 0, s, a); return launch_status();
+          case 3: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 3>), grid, block, 0, s, a); return launch_status();
+          case 7: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 7>), grid, block, 0, s, a); return launch_status();
+          case 15: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 15>), grid, block, 0, s, a); return launch_status();
+          case 16: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 16>), grid, block, 0, s, a); return launch_status();
+          case 8: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 8>), grid, block, 0, s, a); return launch_status();
+          case 4: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 4>), grid, block, 0, s, a); return launch_status();
+          case 32: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 32>), grid, block, 0, s, a); return launch_status();
+          case 39: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 39>), grid, block, 0, s, a); return launch_status();
+          default: break;
+        }
+      }
       hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16>), grid, block, 0, s, a);
       return launch_status();
     }

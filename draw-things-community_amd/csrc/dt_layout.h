@@ -86,6 +86,28 @@ __device__ __forceinline__ void unpack32(const uint32_t (&raw)[Q], uint32_t (&id
     }
   }
 }
+
+// Indices 16*HALF .. 16*HALF + 15 of the same 32-index granule.
+template <int Q, int HALF>
+__device__ __forceinline__ void unpack16(const uint32_t (&raw)[Q], uint32_t (&idx)[16]) {
+  uint32_t be[Q];
+#pragma unroll
+  for (int i = 0; i < Q; i++) be[i] = __builtin_bswap32(raw[i]);
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    const int bit = (16 * HALF + j) * Q;
+    const int word = bit >> 5;
+    const int off = bit & 31;
+    if (off + Q <= 32) {
+      idx[j] = (be[word] >> (32 - off - Q)) & ((1u << Q) - 1);
+    } else {
+      const int sh = 64 - off - Q;
+      const int wn = word + 1 < Q ? word + 1 : word;
+      uint32_t v = __builtin_amdgcn_alignbit(be[word], be[wn], sh);
+      idx[j] = v & ((1u << Q) - 1);
+    }
+  }
+}
 #endif
 
 }  // namespace dt
