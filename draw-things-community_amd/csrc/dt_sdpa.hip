@@ -1,53 +1,65 @@
 // K3: ScaledDotProductAttention, flash-style, fp16 in / fp32 statistics, gfx950.
 //
-// One 256-thread workgroup owns 4 * QB * 32 query rows of one (batch, head);
-// each wave owns QB blocks of 32 rows.  K/V arrive in tiles of 64 keys that
-// are staged through LDS (double-buffered, one barrier per tile).
+// One 512-thread workgroup (8 waves, two per SIMD) owns 256 query rows of one
+// (batch, head); each wave owns 32 of them.  K/V arrive in tiles of 64 keys,
+// staged row-major through LDS (double-buffered, one barrier per tile).
 //
 // Everything is computed transposed so that the query index is the MFMA
 // column (lane & 31) in every stage:
 //   S^T = K Q^T          A = K tile rows from LDS, B = Q^T held in registers
-//   O^T = V^T P^T        A = V^T from LDS,         B = P^T = the S^T accumulator
+//   O^T = V^T P^T        A = V^T, B = P^T = the S^T accumulator itself
 // The accumulator of a 32x32 MFMA holds, for column q = lane & 31, rows
 // 8*(v/4) + 4*(lane/32) + (v%4), v = 0..15.  Feeding it back as the B operand
-// only permutes the summation index, so the V^T operand is read from LDS with
-// the same permutation and P never leaves registers.  The softmax row
-// reductions are therefore in-lane plus one exchange with lane ^ 32.
+// only permutes the summation index, so the V^T operand is fetched with the
+// same permutation and P never leaves registers; the softmax row reductions
+// are in-lane plus one exchange with lane ^ 32.  V stays row-major in LDS:
+// the V^T operand (head dimension along lanes, keys along registers) comes
+// from ds_read_b64_tr_b16, which hands lane j of a 16-lane group the element
+// column (j % 4) of the rows addressed by lanes (j / 4) + {0, 4, 8, 12}.
 #include "dt_common.h"
 #include "dt_sdpa.h"
 
 namespace dt {
 
-constexpr int BKV = 64;  // keys per tile
+constexpr int BKV = 64;     // keys per tile
+constexpr int QWAVES = 8;   // waves per workgroup, 32 query rows each
+constexpr int QROWS = QWAVES * 32;
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
-// V^T tile in LDS: row d holds 64 keys as 16 units of 4 keys (8 bytes); unit u
-// of row d is stored at unit u ^ f(d).  Writers (fixed key group, d = 8*g + j
-// over 16 lanes) and readers (fixed unit, 16 consecutive d) both hit 16
-// distinct units, i.e. all 32 banks once.
-__device__ __forceinline__ int vt_swz(int d) { return (d & 15) ^ ((d >> 4) & 7); }
-
+// LDS layouts (measured bank-conflict free on this part: 64 banks, 16 lanes of
+// a 16-byte access or 32 lanes of an 8-byte access per clock).
+// K tile: [64 keys][DP] halfs; 16-byte chunk c of key row r is stored at a
+// swizzled chunk so that 16 consecutive rows of one chunk column spread over
+// all banks.
 template <int DP>
-struct SdpaSmem {
-  static constexpr int KROW = DP + 8;  // halfs; 16 extra bytes per row spread 16-byte reads of 8 consecutive keys over all banks
-  half_t k[2][BKV * KROW];
-  half_t vt[2][DP * BKV];
-};
+__device__ __forceinline__ int k_chunk_swz(int row, int c) {
+  if constexpr (DP == 128) return c ^ (row & 15);
+  return c ^ ((row >> 1) & 7);
+}
+// V tile: [64 keys][DP] halfs; the transposing read touches 4 consecutive key
+// rows x 64 contiguous bytes per 32 lanes, so 64-byte units are swizzled over
+// the row index.
+template <int DP>
+__device__ __forceinline__ int v_unit_swz(int row, int u) {
+  if constexpr (DP == 128) return u ^ (row & 3);
+  return u ^ ((row >> 1) & 1);
+}
 
-template <int DP, int QB>
-__global__ void __launch_bounds__(256) sdpa_kernel(const SdpaArgs a) {
-  constexpr int KROW = SdpaSmem<DP>::KROW;
-  constexpr int DCH = DP / 8;                 // 16-byte chunks per row
-  constexpr int K_LOADS = BKV * DCH / 256;    // per thread per tile (4 at DP = 128)
-  constexpr int V_TASKS = (BKV / 4) * DCH;    // 4-key x 8-d transposes per tile
-  constexpr int DB = DP / 32;                 // 32-wide blocks of the head dimension
-  constexpr int KS = DP / 16;                 // MFMA k-steps over the head dimension
-  constexpr int QROWS = 4 * QB * 32;
+template <int DP, bool PREMUL>
+__global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
+  constexpr int ROWB = DP * 2;                 // bytes per tile row
+  constexpr int DCH = DP / 8;                  // 16-byte chunks per row
+  constexpr int TILE_B = BKV * ROWB;           // bytes of one K (or V) tile
+  constexpr int LOADS = BKV * DCH / 512;       // 16-byte chunks per thread per tile (2 at DP = 128)
+  constexpr int DB = DP / 32;                  // 32-wide blocks of the head dimension
+  constexpr int KS = DP / 16;                  // MFMA k-steps over the head dimension
+  static_assert(LOADS >= 1, "tile");
 
-  __shared__ __attribute__((aligned(16))) SdpaSmem<DP> sm;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * TILE_B];  // [stage][K | V]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -72,10 +84,9 @@ __global__ void __launch_bounds__(256) sdpa_kernel(const SdpaArgs a) {
 
   // ---- Q^T fragments straight from global memory -----------------------
   // B operand of K Q^T: lane holds query column l32, head-dim slots 16*ks + 8*hi + 0..7.
-  half8_t qf[QB][KS];
-#pragma unroll
-  for (int qb = 0; qb < QB; qb++) {
-    int64_t qi = (int64_t)qt * QROWS + (wave * QB + qb) * 32 + l32;
+  half8_t qf[KS];
+  {
+    int64_t qi = (int64_t)qt * QROWS + wave * 32 + l32;
     if (qi >= Sq) qi = Sq - 1;
     int sg = 0;
 #pragma unroll
@@ -87,15 +98,20 @@ __global__ void __launch_bounds__(256) sdpa_kernel(const SdpaArgs a) {
       const int d0 = ks * 16 + hi * 8;
       uint4_t v = uint4_t{0, 0, 0, 0};
       if (d0 < D) v = *reinterpret_cast<const uint4_t*>(qp + d0);
-      qf[qb][ks] = __builtin_bit_cast(half8_t, v);
+      qf[ks] = __builtin_bit_cast(half8_t, v);
     }
   }
 
   // ---- K / V tile loaders ------------------------------------------------
-  uint4_t k_reg[K_LOADS];
-  uint4_t v_reg[4];
-  const bool v_on = tid < V_TASKS;
-  const int v_kg = tid / DCH, v_dg = tid % DCH;
+  uint4_t k_reg[LOADS], v_reg[LOADS];
+  int k_dst[LOADS], v_dst[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; i++) {
+    const int c = tid + i * 512;
+    const int row = c / DCH, ch = c % DCH;
+    k_dst[i] = row * ROWB + k_chunk_swz<DP>(row, ch) * 16;
+    v_dst[i] = row * ROWB + v_unit_swz<DP>(row, ch >> 2) * 64 + (ch & 3) * 16;
+  }
 
   auto kv_row_ptr = [&](const SdpaSeg* segs, int64_t kj) -> const uint16_t* {
     int sg = 0;
@@ -107,64 +123,56 @@ __global__ void __launch_bounds__(256) sdpa_kernel(const SdpaArgs a) {
 
   auto issue_kv = [&](int64_t j0) {
 #pragma unroll
-    for (int i = 0; i < K_LOADS; i++) {
-      const int c = tid + i * 256;
-      const int row = c / DCH, dc = c % DCH;
+    for (int i = 0; i < LOADS; i++) {
+      const int c = tid + i * 512;
+      const int row = c / DCH, ch = c % DCH;
       const int64_t kj = j0 + row;
-      uint4_t v = uint4_t{0, 0, 0, 0};
-      if (kj < Skv && dc * 8 < D) v = *reinterpret_cast<const uint4_t*>(kv_row_ptr(a.k, kj) + dc * 8);
-      k_reg[i] = v;
-    }
-    if (v_on) {
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int64_t kj = j0 + v_kg * 4 + i;
-        uint4_t v = uint4_t{0, 0, 0, 0};  // rows past the end must be zero: 0 * garbage could be NaN
-        if (kj < Skv && v_dg * 8 < D) v = *reinterpret_cast<const uint4_t*>(kv_row_ptr(a.v, kj) + v_dg * 8);
-        v_reg[i] = v;
+      uint4_t kv = uint4_t{0, 0, 0, 0}, vv = uint4_t{0, 0, 0, 0};  // rows past the end must be zero: 0 * garbage could be NaN
+      if (kj < Skv && ch * 8 < D) {
+        kv = *reinterpret_cast<const uint4_t*>(kv_row_ptr(a.k, kj) + ch * 8);
+        vv = *reinterpret_cast<const uint4_t*>(kv_row_ptr(a.v, kj) + ch * 8);
       }
+      k_reg[i] = kv;
+      v_reg[i] = vv;
     }
   };
-
   auto stage_kv = [&](int st) {
+    unsigned char* kb = smem + st * 2 * TILE_B;
+    unsigned char* vb = kb + TILE_B;
 #pragma unroll
-    for (int i = 0; i < K_LOADS; i++) {
-      const int c = tid + i * 256;
-      const int row = c / DCH, dc = c % DCH;
-      *reinterpret_cast<uint4_t*>(&sm.k[st][row * KROW + dc * 8]) = k_reg[i];
-    }
-    if (v_on) {
-      // 4 keys x 8 d in registers -> 8 rows of V^T, 4 keys (8 bytes) each
-#pragma unroll
-      for (int jj = 0; jj < 4; jj++) {
-        // dword jj of each key row holds d = 2*jj, 2*jj + 1
-        const uint32_t r0 = v_reg[0][jj], r1 = v_reg[1][jj], r2 = v_reg[2][jj], r3 = v_reg[3][jj];
-        const uint32_t lo01 = __builtin_amdgcn_perm(r1, r0, 0x05040100);  // (k0.lo, k1.lo)
-        const uint32_t lo23 = __builtin_amdgcn_perm(r3, r2, 0x05040100);
-        const uint32_t hi01 = __builtin_amdgcn_perm(r1, r0, 0x07060302);  // (k0.hi, k1.hi)
-        const uint32_t hi23 = __builtin_amdgcn_perm(r3, r2, 0x07060302);
-        const int d_even = v_dg * 8 + 2 * jj;
-        const int d_odd = d_even + 1;
-        *reinterpret_cast<uint2_t*>(&sm.vt[st][d_even * BKV + ((v_kg ^ vt_swz(d_even)) << 2)]) = uint2_t{lo01, lo23};
-        *reinterpret_cast<uint2_t*>(&sm.vt[st][d_odd * BKV + ((v_kg ^ vt_swz(d_odd)) << 2)]) = uint2_t{hi01, hi23};
-      }
+    for (int i = 0; i < LOADS; i++) {
+      *reinterpret_cast<uint4_t*>(kb + k_dst[i]) = k_reg[i];
+      *reinterpret_cast<uint4_t*>(vb + v_dst[i]) = v_reg[i];
     }
   };
 
-  // ---- running state -----------------------------------------------------
-  float16_t oacc[QB][DB];
-  float m_run[QB], l_run[QB];
+  // ---- per-lane LDS read offsets --------------------------------------------
+  // K operand: key row kb*32 + l32, chunk 2*ks + hi
+  int k_rd[KS];
 #pragma unroll
-  for (int qb = 0; qb < QB; qb++) {
-    m_run[qb] = -INFINITY;
-    l_run[qb] = 0.f;
+  for (int ks = 0; ks < KS; ks++) k_rd[ks] = l32 * ROWB + k_chunk_swz<DP>(l32, 2 * ks + hi) * 16;
+  // V^T operand through the transposing read: lane i of a 16-lane group addresses
+  // key row (i / 4) of a 4-key run and 4 head-dim elements at 4 * (i % 4); the
+  // two groups of a half-wave cover head-dim 0..15 and 16..31 of block db.
+  const int li = lane & 15, dg = (lane >> 4) & 1;
+  int v_rd[DB];
 #pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-      for (int v = 0; v < 16; v++) oacc[qb][db][v] = 0.f;
+  for (int db = 0; db < DB; db++) {
+    const int row = 4 * hi + (li >> 2);  // + multiples of 4 per k-step: the swizzle depends on row & 3 (or (row >> 1) & 1) only
+    v_rd[db] = row * ROWB + v_unit_swz<DP>(row, db) * 64 + dg * 32 + (li & 3) * 8;
   }
 
-  const float c = a.scale_log2e;
+  // ---- running state -----------------------------------------------------
+  float16_t oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) oacc[db][v] = 0.f;
+  float m_ref = -INFINITY;  // reference for the exponentials (raw score units); trails the true running maximum
+  float l_run = 0.f;        // this lane's share of the row sum
+
+  const float c = PREMUL ? 1.0f : a.scale_log2e;
+  const float thr = 8.0f / c;  // rescale only when the maximum grows by more than 2^8
   const int n_tiles = (int)((Skv + BKV - 1) / BKV);
 
   issue_kv(0);
@@ -175,70 +183,71 @@ __global__ void __launch_bounds__(256) sdpa_kernel(const SdpaArgs a) {
     const int cur = t & 1;
     const bool more = t + 1 < n_tiles;
     if (more) issue_kv((int64_t)(t + 1) * BKV);
+    const unsigned char* kt = smem + cur * 2 * TILE_B;
+    const unsigned char* vt = kt + TILE_B;
 
     // ---- S^T = K Q^T ------------------------------------------------------
-    float16_t sacc[QB][2];
+    float16_t sacc[2];
 #pragma unroll
-    for (int qb = 0; qb < QB; qb++)
+    for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) sacc[qb][kb][v] = 0.f;
+      for (int v = 0; v < 16; v++) sacc[kb][v] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
 #pragma unroll
       for (int kb = 0; kb < 2; kb++) {
-        const half8_t kf =
-            *reinterpret_cast<const half8_t*>(&sm.k[cur][(kb * 32 + l32) * KROW + ks * 16 + hi * 8]);
-#pragma unroll
-        for (int qb = 0; qb < QB; qb++)
-          sacc[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[qb][ks], sacc[qb][kb], 0, 0, 0);
+        const half8_t kf = *reinterpret_cast<const half8_t*>(kt + kb * 32 * ROWB + k_rd[ks]);
+        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], sacc[kb], 0, 0, 0);
       }
     }
 
     // ---- online softmax (per query column, statistics in fp32) -----------
     const bool ragged = (int64_t)(t + 1) * BKV > Skv;
-    half8_t pf[QB][2][2];
-#pragma unroll
-    for (int qb = 0; qb < QB; qb++) {
-      float mx = -INFINITY;
+    if (PREMUL || ragged) {
 #pragma unroll
       for (int kb = 0; kb < 2; kb++)
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-          float s = sacc[qb][kb][v] * c;
+          float s = sacc[kb][v];
+          if (PREMUL) s *= a.scale_log2e;
           if (ragged) {
             const int64_t kj = (int64_t)t * BKV + kb * 32 + 8 * (v >> 2) + 4 * hi + (v & 3);
             if (kj >= Skv) s = -INFINITY;
           }
-          sacc[qb][kb][v] = s;
-          mx = fmaxf(mx, s);
+          sacc[kb][v] = s;
         }
-      mx = fmaxf(mx, xor32(mx));
-      const float m_new = fmaxf(m_run[qb], mx);
-      const float alpha = fast_exp2(m_run[qb] - m_new);  // first tile: exp2(-inf) = 0
-      m_run[qb] = m_new;
-      float psum = 0.f;
+    }
+    float mx = sacc[0][0];
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++)
+    for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-          const float p = fast_exp2(sacc[qb][kb][v] - m_new);
-          sacc[qb][kb][v] = p;
-          psum += p;
-        }
-      l_run[qb] = l_run[qb] * alpha + psum;
+      for (int v = (kb == 0 ? 1 : 0); v < 16; v++) mx = fmaxf(mx, sacc[kb][v]);
+    mx = fmaxf(mx, xor32(mx));
+    if (__builtin_amdgcn_ballot_w64(mx > m_ref + thr) != 0) {
+      // some row's maximum moved far enough: move every row's reference up to its running maximum
+      const float m_new = fmaxf(m_ref, mx);
+      const float alpha = fast_exp2((m_ref - m_new) * c);  // first tile: exp2(-inf) = 0
+      m_ref = m_new;
+      l_run *= alpha;
 #pragma unroll
       for (int db = 0; db < DB; db++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) oacc[qb][db][v] *= alpha;
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-          for (int e = 0; e < 8; e++) pf[qb][kb][tt][e] = (half_t)sacc[qb][kb][8 * tt + e];
+        for (int v = 0; v < 16; v++) oacc[db][v] *= alpha;
     }
+    const float mc = m_ref * c;
+    float psum = 0.f;
+    half8_t pf[2][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+      for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const float p = fast_exp2(__builtin_fmaf(sacc[kb][8 * tt + e], c, -mc));
+          psum += p;
+          pf[kb][tt][e] = (half_t)p;
+        }
+    l_run += psum;
 
     // ---- O^T += V^T P^T ----------------------------------------------------
     // k-slot e of lane half `hi` in step (kb, tt) is key kb*32 + 16*tt + 8*(e/4) + 4*hi + (e%4)
@@ -246,17 +255,15 @@ __global__ void __launch_bounds__(256) sdpa_kernel(const SdpaArgs a) {
     for (int kb = 0; kb < 2; kb++)
 #pragma unroll
       for (int tt = 0; tt < 2; tt++) {
-        const int u0 = (kb * 32 + 16 * tt) / 4 + hi;  // unit of keys base + 4*hi .. +3
+        const int koff = (kb * 32 + 16 * tt) * ROWB;
 #pragma unroll
         for (int db = 0; db < DB; db++) {
-          const int d = db * 32 + l32;
-          const int sw = vt_swz(d);
-          const half4_t lo = *reinterpret_cast<const half4_t*>(&sm.vt[cur][d * BKV + ((u0 ^ sw) << 2)]);
-          const half4_t hi4 = *reinterpret_cast<const half4_t*>(&sm.vt[cur][d * BKV + (((u0 + 2) ^ sw) << 2)]);
-          const half8_t vf = half8_t{lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-#pragma unroll
-          for (int qb = 0; qb < QB; qb++)
-            oacc[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[qb][kb][tt], oacc[qb][db], 0, 0, 0);
+          typedef __attribute__((address_space(3))) short4_t lds_s4;
+          const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt + koff + v_rd[db]));
+          const short4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt + koff + 8 * ROWB + v_rd[db]));
+          typedef short short8_t __attribute__((ext_vector_type(8)));
+          const short8_t v8 = short8_t{lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, v8), pf[kb][tt], oacc[db], 0, 0, 0);
         }
       }
 
@@ -265,44 +272,66 @@ __global__ void __launch_bounds__(256) sdpa_kernel(const SdpaArgs a) {
   }
 
   // ---- normalise and store O ----------------------------------------------
-#pragma unroll
-  for (int qb = 0; qb < QB; qb++) {
-    const int64_t qi = (int64_t)qt * QROWS + (wave * QB + qb) * 32 + l32;
-    const float l_tot = l_run[qb] + xor32(l_run[qb]);
+  // O^T block db: lane holds query column l32 and head-dim 8*g + 4*hi + (0..3);
+  // swapping the odd groups of the low half-wave with the even groups of the
+  // high half-wave leaves every lane with runs of 8 consecutive head-dim
+  // elements (16-byte stores).
+  {
+    const int64_t qi = (int64_t)qt * QROWS + wave * 32 + l32;
+    const float l_tot = l_run + xor32(l_run);
     const float inv = 1.0f / l_tot;
-    if (qi >= Sq) continue;
-    uint16_t* op = a.o + b * a.o_sb + qi * a.o_ss + h * a.o_sh;
+    uint16_t* op = a.o + b * a.o_sb + (qi < Sq ? qi : 0) * a.o_ss + h * a.o_sh;
+    const bool vec_ok = ((a.o_sb | a.o_ss | a.o_sh) & 7) == 0 && (reinterpret_cast<uintptr_t>(a.o) & 15) == 0;
 #pragma unroll
-    for (int db = 0; db < DB; db++)
+    for (int db = 0; db < DB; db++) {
+      uint32_t pk[4][2];
 #pragma unroll
       for (int g = 0; g < 4; g++) {
-        const int d0 = db * 32 + 8 * g + 4 * hi;
-        if (d0 < D) {
-          half4_t o4;
+        pk[g][0] = (uint32_t)half_to_bits((half_t)(oacc[db][4 * g] * inv)) |
+                   ((uint32_t)half_to_bits((half_t)(oacc[db][4 * g + 1] * inv)) << 16);
+        pk[g][1] = (uint32_t)half_to_bits((half_t)(oacc[db][4 * g + 2] * inv)) |
+                   ((uint32_t)half_to_bits((half_t)(oacc[db][4 * g + 3] * inv)) << 16);
+      }
 #pragma unroll
-          for (int e = 0; e < 4; e++) o4[e] = (half_t)(oacc[qb][db][4 * g + e] * inv);
-          *reinterpret_cast<half4_t*>(op + d0) = o4;
+      for (int gp = 0; gp < 2; gp++) {
+        uint32_t run[4];
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+          auto r = __builtin_amdgcn_permlane32_swap(pk[2 * gp][e], pk[2 * gp + 1][e], false, false);
+          run[e] = r[0];
+          run[2 + e] = r[1];
+        }
+        const int d0 = db * 32 + 16 * gp + 8 * hi;
+        if (qi < Sq && d0 < D) {
+          if (vec_ok) {
+            *reinterpret_cast<uint4_t*>(op + d0) = uint4_t{run[0], run[1], run[2], run[3]};
+          } else {
+            *reinterpret_cast<uint2_t*>(op + d0) = uint2_t{run[0], run[1]};
+            *reinterpret_cast<uint2_t*>(op + d0 + 4) = uint2_t{run[2], run[3]};
+          }
         }
       }
+    }
   }
 }
 
-template <int DP, int QB>
+template <int DP>
 static dt_status launch(hipStream_t s, SdpaArgs a) {
-  const int qrows = 4 * QB * 32;
-  a.q_tiles = (int)((a.Sq + qrows - 1) / qrows);
+  a.q_tiles = (int)((a.Sq + QROWS - 1) / QROWS);
   int64_t total = (int64_t)a.q_tiles * a.Hq * a.B;
   if (total > 0x7fffffff) return DT_NO_KERNEL;
   a.total_blocks = (int)total;
-  hipLaunchKernelGGL((sdpa_kernel<DP, QB>), dim3((unsigned)total), dim3(256), 0, s, a);
+  if (a.scale_log2e > 0.f && a.scale_log2e < 1e30f)
+    hipLaunchKernelGGL((sdpa_kernel<DP, false>), dim3((unsigned)total), dim3(512), 0, s, a);
+  else
+    hipLaunchKernelGGL((sdpa_kernel<DP, true>), dim3((unsigned)total), dim3(512), 0, s, a);
   return launch_status();
 }
 
 dt_status sdpa_launch(hipStream_t s, const SdpaArgs& a) {
   if (a.B <= 0 || a.Sq <= 0) return DT_OK;
-  const bool big = a.Sq >= 2048;
-  if (a.D <= 64) return big ? launch<64, 2>(s, a) : launch<64, 1>(s, a);
-  return big ? launch<128, 2>(s, a) : launch<128, 1>(s, a);
+  if (a.D <= 64) return launch<64>(s, a);
+  return launch<128>(s, a);
 }
 
 }  // namespace dt
