@@ -28,7 +28,29 @@ constexpr int QROWS = QWAVES * 32;
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+// Combine the two half-waves (lanes l and l ^ 32 hold the same query) without touching LDS:
+// v_permlane32_swap of a register with a copy of itself leaves {low, low} and {high, high}.
+__device__ __forceinline__ void halves32(float v, float& lo, float& hi) {
+  uint32_t a = __builtin_bit_cast(uint32_t, v), b = a;
+  asm volatile("" : "+v"(b));  // the swap needs two distinct registers
+  auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  uint32_t x0 = r[0], x1 = r[1];
+  // keeps the two results apart: without it the compiler has been seen to
+  // combine r[0] with itself when both inputs carry the same value
+  asm volatile("" : "+v"(x0), "+v"(x1));
+  lo = __builtin_bit_cast(float, x0);
+  hi = __builtin_bit_cast(float, x1);
+}
+__device__ __forceinline__ float max32(float v) {
+  float lo, hi;
+  halves32(v, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float sum32(float v) {
+  float lo, hi;
+  halves32(v, lo, hi);
+  return lo + hi;
+}
 
 // LDS layouts (measured bank-conflict free on this part: 64 banks, 16 lanes of
 // a 16-byte access or 32 lanes of an 8-byte access per clock).
@@ -192,17 +214,30 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     for (int kb = 0; kb < 2; kb++)
 #pragma unroll
       for (int v = 0; v < 16; v++) sacc[kb][v] = 0.f;
+    // K fragments are read two k-steps (4 reads) ahead of the MFMAs that use them
+    {
+      half8_t kf[2][4];
+      auto read_k = [&](int buf, int g) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
+        for (int u = 0; u < 4; u++)
+          kf[buf][u] = *reinterpret_cast<const half8_t*>(kt + (u & 1) * 32 * ROWB + k_rd[2 * g + (u >> 1)]);
+      };
+      read_k(0, 0);
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++) {
-        const half8_t kf = *reinterpret_cast<const half8_t*>(kt + kb * 32 * ROWB + k_rd[ks]);
-        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], sacc[kb], 0, 0, 0);
+      for (int g = 0; g < KS / 2; g++) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (g + 1 < KS / 2) read_k((g + 1) & 1, g + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+          sacc[u & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[g & 1][u], qf[2 * g + (u >> 1)], sacc[u & 1], 0, 0, 0);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- online softmax (per query column, statistics in fp32) -----------
-    const bool ragged = (int64_t)(t + 1) * BKV > Skv;
+    const int rem = (int)(Skv - (int64_t)t * BKV);  // keys left, this tile included
+    const bool ragged = rem < BKV;
     if (PREMUL || ragged) {
 #pragma unroll
       for (int kb = 0; kb < 2; kb++)
@@ -211,8 +246,8 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
           float s = sacc[kb][v];
           if (PREMUL) s *= a.scale_log2e;
           if (ragged) {
-            const int64_t kj = (int64_t)t * BKV + kb * 32 + 8 * (v >> 2) + 4 * hi + (v & 3);
-            if (kj >= Skv) s = -INFINITY;
+            const int kj = kb * 32 + 8 * (v >> 2) + 4 * hi + (v & 3);
+            if (kj >= rem) s = -INFINITY;
           }
           sacc[kb][v] = s;
         }
@@ -222,7 +257,7 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     for (int kb = 0; kb < 2; kb++)
 #pragma unroll
       for (int v = (kb == 0 ? 1 : 0); v < 16; v++) mx = fmaxf(mx, sacc[kb][v]);
-    mx = fmaxf(mx, xor32(mx));
+    mx = max32(mx);
     if (__builtin_amdgcn_ballot_w64(mx > m_ref + thr) != 0) {
       // some row's maximum moved far enough: move every row's reference up to its running maximum
       const float m_new = fmaxf(m_ref, mx);
@@ -251,21 +286,34 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
 
     // ---- O^T += V^T P^T ----------------------------------------------------
     // k-slot e of lane half `hi` in step (kb, tt) is key kb*32 + 16*tt + 8*(e/4) + 4*hi + (e%4)
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-      for (int tt = 0; tt < 2; tt++) {
-        const int koff = (kb * 32 + 16 * tt) * ROWB;
+    // V^T fragments of the next 16-key step are read while the current step's MFMAs run
+    {
+      typedef __attribute__((address_space(3))) short4_t lds_s4;
+      typedef short short8_t __attribute__((ext_vector_type(8)));
+      short4_t vlo[2][DB], vhi[2][DB];
+      auto read_v = [&](int buf, int step) {
+        const int koff = 16 * step * ROWB;
 #pragma unroll
         for (int db = 0; db < DB; db++) {
-          typedef __attribute__((address_space(3))) short4_t lds_s4;
-          const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt + koff + v_rd[db]));
-          const short4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt + koff + 8 * ROWB + v_rd[db]));
-          typedef short short8_t __attribute__((ext_vector_type(8)));
-          const short8_t v8 = short8_t{lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, v8), pf[kb][tt], oacc[db], 0, 0, 0);
+          vlo[buf][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt + koff + v_rd[db]));
+          vhi[buf][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt + koff + 8 * ROWB + v_rd[db]));
+        }
+      };
+      read_v(0, 0);
+#pragma unroll
+      for (int step = 0; step < 4; step++) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (step + 1 < 4) read_v((step + 1) & 1, step + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+          const short4_t lo = vlo[step & 1][db], h4 = vhi[step & 1][db];
+          const short8_t v8 = short8_t{lo[0], lo[1], lo[2], lo[3], h4[0], h4[1], h4[2], h4[3]};
+          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, v8), pf[step >> 1][step & 1], oacc[db], 0, 0, 0);
         }
       }
+      __builtin_amdgcn_sched_barrier(0);
+    }
 
     if (more) stage_kv(cur ^ 1);
     __syncthreads();
@@ -278,7 +326,7 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   // elements (16-byte stores).
   {
     const int64_t qi = (int64_t)qt * QROWS + wave * 32 + l32;
-    const float l_tot = l_run + xor32(l_run);
+    const float l_tot = sum32(l_run);
     const float inv = 1.0f / l_tot;
     uint16_t* op = a.o + b * a.o_sb + (qi < Sq ? qi : 0) * a.o_ss + h * a.o_sh;
     const bool vec_ok = ((a.o_sb | a.o_ss | a.o_sh) & 7) == 0 && (reinterpret_cast<uintptr_t>(a.o) & 15) == 0;
