@@ -81,7 +81,7 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   constexpr int KS = DP / 16;                  // MFMA k-steps over the head dimension
   static_assert(LOADS >= 1, "tile");
 
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * TILE_B];  // [stage][K | V]
+  __shared__ __attribute__((aligned(16))) unsigned char smem[4 * TILE_B];  // K stage 0, K stage 1, V stage 0, V stage 1
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -125,47 +125,83 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   }
 
   // ---- K / V tile loaders ------------------------------------------------
-  uint4_t k_reg[LOADS], v_reg[LOADS];
-  int k_dst[LOADS], v_dst[LOADS];
+  // Each thread moves LOADS 16-byte chunks of every K tile and of every V tile.
+  // Row pointers advance by 64 rows per tile; they are re-derived from the
+  // segment table only when a row leaves its segment.
+  int k_dst[LOADS], v_dst[LOADS], ld_row[LOADS], ld_ch[LOADS];
 #pragma unroll
   for (int i = 0; i < LOADS; i++) {
     const int c = tid + i * 512;
     const int row = c / DCH, ch = c % DCH;
+    ld_row[i] = row;
+    ld_ch[i] = ch;
     k_dst[i] = row * ROWB + k_chunk_swz<DP>(row, ch) * 16;
     v_dst[i] = row * ROWB + v_unit_swz<DP>(row, ch >> 2) * 64 + (ch & 3) * 16;
   }
-
-  auto kv_row_ptr = [&](const SdpaSeg* segs, int64_t kj) -> const uint16_t* {
+  struct RowPtr {
+    const uint16_t* p;  // chunk address of the current row
+    int64_t row;        // joint row index
+    int64_t end;        // first joint row past the current segment
+    int64_t step;       // elements per 64 rows inside the current segment
+  };
+  auto locate = [&](const SdpaSeg* segs, int64_t kj, int ch, RowPtr& r) {
     int sg = 0;
 #pragma unroll
     for (int i = 1; i < kMaxSeg; i++)
       if (i < a.n_kvseg && kj >= segs[i].start) sg = i;
-    return segs[sg].ptr + b * segs[sg].sb + (kj - segs[sg].start) * segs[sg].ss + hk * segs[sg].sh;
+    r.p = segs[sg].ptr + b * segs[sg].sb + (kj - segs[sg].start) * segs[sg].ss + hk * segs[sg].sh + ch * 8;
+    r.row = kj;
+    r.end = (sg + 1 < a.n_kvseg) ? segs[sg + 1].start : Skv;
+    r.step = segs[sg].ss * BKV;
   };
-
-  auto issue_kv = [&](int64_t j0) {
+  auto advance = [&](const SdpaSeg* segs, int ch, RowPtr& r) {
+    const int64_t kj = r.row + BKV;
+    if (kj < r.end) {
+      r.row = kj;
+      r.p += r.step;
+    } else if (kj < Skv) {
+      locate(segs, kj, ch, r);
+    } else {
+      r.row = kj;
+    }
+  };
+  RowPtr kp[LOADS], vp[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; i++) {
+    locate(a.k, ld_row[i] < Skv ? ld_row[i] : 0, ld_ch[i], kp[i]);
+    kp[i].row = ld_row[i];
+    locate(a.v, ld_row[i] < Skv ? ld_row[i] : 0, ld_ch[i], vp[i]);
+    vp[i].row = ld_row[i];
+  }
+  uint4_t k_reg[LOADS], v_reg[LOADS];
+  // loads the K (or V) tile the pointers stand on, then moves them to the next tile
+  auto issue_k = [&]() {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
-      const int c = tid + i * 512;
-      const int row = c / DCH, ch = c % DCH;
-      const int64_t kj = j0 + row;
-      uint4_t kv = uint4_t{0, 0, 0, 0}, vv = uint4_t{0, 0, 0, 0};  // rows past the end must be zero: 0 * garbage could be NaN
-      if (kj < Skv && ch * 8 < D) {
-        kv = *reinterpret_cast<const uint4_t*>(kv_row_ptr(a.k, kj) + ch * 8);
-        vv = *reinterpret_cast<const uint4_t*>(kv_row_ptr(a.v, kj) + ch * 8);
-      }
+      uint4_t kv = uint4_t{0, 0, 0, 0};
+      if (kp[i].row < Skv && ld_ch[i] * 8 < D) kv = *reinterpret_cast<const uint4_t*>(kp[i].p);
       k_reg[i] = kv;
-      v_reg[i] = vv;
+      advance(a.k, ld_ch[i], kp[i]);
     }
   };
-  auto stage_kv = [&](int st) {
-    unsigned char* kb = smem + st * 2 * TILE_B;
-    unsigned char* vb = kb + TILE_B;
+  auto issue_v = [&]() {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
-      *reinterpret_cast<uint4_t*>(kb + k_dst[i]) = k_reg[i];
-      *reinterpret_cast<uint4_t*>(vb + v_dst[i]) = v_reg[i];
+      uint4_t vv = uint4_t{0, 0, 0, 0};  // rows past the end must be zero: 0 * garbage could be NaN
+      if (vp[i].row < Skv && ld_ch[i] * 8 < D) vv = *reinterpret_cast<const uint4_t*>(vp[i].p);
+      v_reg[i] = vv;
+      advance(a.v, ld_ch[i], vp[i]);
     }
+  };
+  auto stage_k = [&](int st) {
+    unsigned char* kb = smem + st * TILE_B;
+#pragma unroll
+    for (int i = 0; i < LOADS; i++) *reinterpret_cast<uint4_t*>(kb + k_dst[i]) = k_reg[i];
+  };
+  auto stage_v = [&](int st) {
+    unsigned char* vb = smem + (2 + st) * TILE_B;
+#pragma unroll
+    for (int i = 0; i < LOADS; i++) *reinterpret_cast<uint4_t*>(vb + v_dst[i]) = v_reg[i];
   };
 
   // ---- per-lane LDS read offsets --------------------------------------------
@@ -197,45 +233,38 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   const float thr = 8.0f / c;  // rescale only when the maximum grows by more than 2^8
   const int n_tiles = (int)((Skv + BKV - 1) / BKV);
 
-  issue_kv(0);
-  stage_kv(0);
-  __syncthreads();
+  float16_t sacc[2];   // S^T of the tile in flight (keys x queries)
+  half8_t pf[2][2];    // its probabilities, as the B operand of the second MFMA
 
-  for (int t = 0; t < n_tiles; t++) {
-    const int cur = t & 1;
-    const bool more = t + 1 < n_tiles;
-    if (more) issue_kv((int64_t)(t + 1) * BKV);
-    const unsigned char* kt = smem + cur * 2 * TILE_B;
-    const unsigned char* vt = kt + TILE_B;
-
-    // ---- S^T = K Q^T ------------------------------------------------------
-    float16_t sacc[2];
+  // S^T = K Q^T for the K tile in stage st
+  auto s_phase = [&](int st) {
+    const unsigned char* kt = smem + st * TILE_B;
 #pragma unroll
     for (int kb = 0; kb < 2; kb++)
 #pragma unroll
       for (int v = 0; v < 16; v++) sacc[kb][v] = 0.f;
     // K fragments are read two k-steps (4 reads) ahead of the MFMAs that use them
-    {
-      half8_t kf[2][4];
-      auto read_k = [&](int buf, int g) {
+    half8_t kf[2][4];
+    auto read_k = [&](int buf, int g) {
 #pragma unroll
-        for (int u = 0; u < 4; u++)
-          kf[buf][u] = *reinterpret_cast<const half8_t*>(kt + (u & 1) * 32 * ROWB + k_rd[2 * g + (u >> 1)]);
-      };
-      read_k(0, 0);
+      for (int u = 0; u < 4; u++)
+        kf[buf][u] = *reinterpret_cast<const half8_t*>(kt + (u & 1) * 32 * ROWB + k_rd[2 * g + (u >> 1)]);
+    };
+    read_k(0, 0);
 #pragma unroll
-      for (int g = 0; g < KS / 2; g++) {
-        __builtin_amdgcn_sched_barrier(0);
-        if (g + 1 < KS / 2) read_k((g + 1) & 1, g + 1);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int u = 0; u < 4; u++)
-          sacc[u & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[g & 1][u], qf[2 * g + (u >> 1)], sacc[u & 1], 0, 0, 0);
-      }
+    for (int g = 0; g < KS / 2; g++) {
       __builtin_amdgcn_sched_barrier(0);
+      if (g + 1 < KS / 2) read_k((g + 1) & 1, g + 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+        sacc[u & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[g & 1][u], qf[2 * g + (u >> 1)], sacc[u & 1], 0, 0, 0);
     }
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
-    // ---- online softmax (per query column, statistics in fp32) -----------
+  // online softmax of tile t (per query column, statistics in fp32): sacc -> pf
+  auto softmax_phase = [&](int t) {
     const int rem = (int)(Skv - (int64_t)t * BKV);  // keys left, this tile included
     const bool ragged = rem < BKV;
     if (PREMUL || ragged) {
@@ -271,7 +300,6 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     }
     const float mc = m_ref * c;
     float psum = 0.f;
-    half8_t pf[2][2];
 #pragma unroll
     for (int kb = 0; kb < 2; kb++)
 #pragma unroll
@@ -283,39 +311,74 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
           pf[kb][tt][e] = (half_t)p;
         }
     l_run += psum;
+  };
 
-    // ---- O^T += V^T P^T ----------------------------------------------------
-    // k-slot e of lane half `hi` in step (kb, tt) is key kb*32 + 16*tt + 8*(e/4) + 4*hi + (e%4)
+  // O^T += V^T P^T for the V tile in stage st.
+  // k-slot e of lane half `hi` in 16-key step s is key 16*s + 8*(e/4) + 4*hi + (e%4).
+  auto pv_phase = [&](int st) {
+    const unsigned char* vt = smem + (2 + st) * TILE_B;
+    typedef __attribute__((address_space(3))) short4_t lds_s4;
+    typedef short short8_t __attribute__((ext_vector_type(8)));
     // V^T fragments of the next 16-key step are read while the current step's MFMAs run
-    {
-      typedef __attribute__((address_space(3))) short4_t lds_s4;
-      typedef short short8_t __attribute__((ext_vector_type(8)));
-      short4_t vlo[2][DB], vhi[2][DB];
-      auto read_v = [&](int buf, int step) {
-        const int koff = 16 * step * ROWB;
+    short4_t vlo[2][DB], vhi[2][DB];
+    auto read_v = [&](int buf, int step) {
+      const int koff = 16 * step * ROWB;
 #pragma unroll
-        for (int db = 0; db < DB; db++) {
-          vlo[buf][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt + koff + v_rd[db]));
-          vhi[buf][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt + koff + 8 * ROWB + v_rd[db]));
-        }
-      };
-      read_v(0, 0);
-#pragma unroll
-      for (int step = 0; step < 4; step++) {
-        __builtin_amdgcn_sched_barrier(0);
-        if (step + 1 < 4) read_v((step + 1) & 1, step + 1);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int db = 0; db < DB; db++) {
-          const short4_t lo = vlo[step & 1][db], h4 = vhi[step & 1][db];
-          const short8_t v8 = short8_t{lo[0], lo[1], lo[2], lo[3], h4[0], h4[1], h4[2], h4[3]};
-          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, v8), pf[step >> 1][step & 1], oacc[db], 0, 0, 0);
-        }
+      for (int db = 0; db < DB; db++) {
+        vlo[buf][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt + koff + v_rd[db]));
+        vhi[buf][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt + koff + 8 * ROWB + v_rd[db]));
       }
+    };
+    read_v(0, 0);
+#pragma unroll
+    for (int step = 0; step < 4; step++) {
       __builtin_amdgcn_sched_barrier(0);
+      if (step + 1 < 4) read_v((step + 1) & 1, step + 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const short4_t lo = vlo[step & 1][db], h4 = vhi[step & 1][db];
+        const short8_t v8 = short8_t{lo[0], lo[1], lo[2], lo[3], h4[0], h4[1], h4[2], h4[3]};
+        oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, v8), pf[step >> 1][step & 1], oacc[db], 0, 0, 0);
+      }
     }
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
-    if (more) stage_kv(cur ^ 1);
+  // ---- pipeline ---------------------------------------------------------------
+  // Interval t (between two barriers) has K tile t and V tile t-1 readable in
+  // LDS while K tile t+1 and V tile t are written.  Every wave runs
+  //   O += V(t-1) P(t-1) ;  S(t) = K(t) Q ;  P(t) = softmax(S(t))
+  // per interval -- two MFMA phases back to back, then one VALU phase.  The two
+  // waves of a SIMD (w and w+4) run that cycle half a period apart: the second
+  // one starts each interval with the softmax of the scores it produced in the
+  // previous interval, so one wave's exponentials overlap the other's MFMAs.
+  const bool second = wave >= 4;
+  issue_k();   // K(0)
+  stage_k(0);
+  issue_k();   // K(1)
+  issue_v();   // V(0)
+  __syncthreads();
+
+  for (int t = 0; t <= n_tiles; t++) {
+    // registers hold K(t+1) and V(t): write them, then start K(t+2) and V(t+1)
+    if (t + 1 < n_tiles) stage_k((t + 1) & 1);
+    if (t < n_tiles) stage_v(t & 1);
+    if (t + 2 < n_tiles) issue_k();
+    if (t + 1 < n_tiles) issue_v();
+    if (!second) {
+      if (t > 0) pv_phase((t - 1) & 1);
+      if (t < n_tiles) {
+        s_phase(t & 1);
+        softmax_phase(t);
+      }
+    } else {
+      if (t > 0) {
+        softmax_phase(t - 1);
+        pv_phase((t - 1) & 1);
+      }
+      if (t < n_tiles) s_phase(t & 1);
+    }
     __syncthreads();
   }
 
