@@ -188,28 +188,30 @@ def main():
 
         oracle.build()
         ncores = oracle.C.lib.dto_num_threads()
-        m_s, rows_s, heads_s = 192, 768, 2
-        xs = (rng.standard_normal((m_s, C))).astype(np.float16)
+        # the whole block at full size: 8 Dense (6 QKV + 2 out, per-stream rows) + attention over all heads
         t0 = time.perf_counter()
+        xs_c = rng.standard_normal((T, C)).astype(np.float16)
+        xs_x = rng.standard_normal((HW, C)).astype(np.float16)
+        t0 = time.perf_counter()
+        for name in ("c_q", "c_k", "c_v", "c_o"):
+            oracle.C.dense_qx(xs_c, packed_host[name], qbits, nib, C, None)
         for name in ("x_q", "x_k", "x_v", "x_o"):
-            oracle.C.dense_qx(xs, packed_host[name], qbits, nib, C, None)
+            oracle.C.dense_qx(xs_x, packed_host[name], qbits, nib, C, None)
         t_dense = time.perf_counter() - t0
-        qs = rng.standard_normal((1, rows_s, heads_s, D)).astype(np.float16)
-        ks = rng.standard_normal((1, S, heads_s, D)).astype(np.float16)
-        vs = rng.standard_normal((1, S, heads_s, D)).astype(np.float16)
+        qs = rng.standard_normal((1, S, H, D)).astype(np.float16)
+        ks = rng.standard_normal((1, S, H, D)).astype(np.float16)
+        vs = rng.standard_normal((1, S, H, D)).astype(np.float16)
         t0 = time.perf_counter()
         oracle.C.sdpa(qs, ks, vs, scale)
         t_sdpa = time.perf_counter() - t0
-        f_dense = 2.0 * m_s * C * C * 4
-        f_sdpa = 4.0 * heads_s * rows_s * S * D
-        # time for the whole block at the sample's rates, then block FLOPs over it
-        t_block = t_dense * (flop_dense / f_dense) + t_sdpa * (flop_sdpa / f_sdpa)
+        t_block = t_dense + t_sdpa
         cpu = {
             "value": round(flop_block / t_block / 1e12, 5), "unit": "TFLOP/s", "cores": int(ncores), "kind": "port",
-            "sample": f"oracle (C, OpenMP): 4 q6p Dense 3072->3072 on {m_s} rows ({t_dense:.2f} s, depalettize included) + "
-                      f"attention of {rows_s} query rows x {heads_s} heads against all {S} keys ({t_sdpa:.2f} s); "
-                      "block time extrapolated linearly in rows/heads",
-            "dense_gflops": round(f_dense / t_dense / 1e9, 1), "sdpa_gflops": round(f_sdpa / t_sdpa / 1e9, 1),
+            "sample": f"oracle (C, OpenMP, {ncores} threads), the whole block at full size, one pass: 8 q6p Dense "
+                      f"3072->3072 (512 / 4096 rows, depalettize included, {t_dense:.2f} s) + attention 24 heads x 4608 x 4608 "
+                      f"({t_sdpa:.2f} s); RMSNorm/RoPE not included",
+            "ms_per_block": round(t_block * 1e3, 1),
+            "dense_gflops": round(flop_dense / t_dense / 1e9, 1), "sdpa_gflops": round(flop_sdpa / t_sdpa / 1e9, 1),
         }
 
     line = {

@@ -12,7 +12,6 @@
 // K-tile and the unpack VALU/LDS work overlaps the matrix pipe.
 #include "dt_common.h"
 #include "dt_layout.h"
-#include <cstdlib>
 
 namespace dt {
 
@@ -82,7 +81,7 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 // eight run MFMAs on a (BN/2) x (BM/4) slice.  The accumulators are held
 // transposed (rows = output features n, columns = tokens m) so that each lane
 // ends up with runs of consecutive n for one token: 16-byte stores.
-template <int Q, int BM, int BN, int MODE, int EXP = 0>
+template <int Q, int BM, int BN, int MODE>
 __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   constexpr int WN = BN / 2, WM = BM / 4;   // per-wave slice: WN features x WM tokens
   constexpr int TN = WN / 32, TM = WM / 32;
@@ -320,11 +319,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     for (int i = 0; i < TN; i++)
 #pragma unroll
       for (int j = 0; j < TM; j++)
-        if constexpr (EXP & 32) {
-          asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fw[buf][i]), "v"(fx[buf][j]));
-        } else {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[buf][i], fx[buf][j], acc[i][j], 0, 0, 0);
-        }
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[buf][i], fx[buf][j], acc[i][j], 0, 0, 0);
   };
 
   // ---- prologue: tiles 0 and 1 into the ring, tiles 2 and 3 in flight ---------
@@ -357,7 +352,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     const int s_cur = t % NST;
     const int s_nxt = (t + 1) % NST;
     const int s_fill = (t + 2) % NST;
-    if constexpr (!(EXP & 1)) issue_loads(Rload);
+    issue_loads(Rload);
     if constexpr (MODE == kPalRow) {
       const int k2 = ((t + 2 + rot) % nk) * BK;
       if (t + 2 < nk && k2 % a.nib == 0) {
@@ -367,21 +362,21 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       }
     }
     if (second) {
-      if constexpr (!(EXP & 2)) stage_to_lds(Rstage, s_fill);
+      stage_to_lds(Rstage, s_fill);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (!(EXP & 8)) read_frags(1, s_cur, 1);
+    read_frags(1, s_cur, 1);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (!(EXP & 16)) mfma_step(0);
+    mfma_step(0);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (!(EXP & 8)) read_frags(0, s_nxt, 0);
+    read_frags(0, s_nxt, 0);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (!(EXP & 16)) mfma_step(1);
+    mfma_step(1);
     __builtin_amdgcn_sched_barrier(0);
     if (!second) {
-      if constexpr (!(EXP & 2)) stage_to_lds(Rstage, s_fill);
+      stage_to_lds(Rstage, s_fill);
     }
-    if constexpr (!(EXP & 4)) __syncthreads();
+    __syncthreads();
   };
 
   // tile T travels in register set T % 3: iteration t stages set (t+2) % 3 and refills set (t+1) % 3
@@ -511,23 +506,6 @@ static dt_status launch_tiled_q(hipStream_t s, const DenseArgs& a, int qbits, in
     case 8: return launch_tiled<8, BM, BN>(s, a, mode);
     case 16: {
       dim3 grid((unsigned)(a.tiles_m * a.tiles_n)), block(512);
-      const char* ex = getenv("DT_DENSE_EXP");
-      int e = ex ? atoi(ex) : 0;
-      if constexpr (BM == 256) {
-        switch (e) {
-          case 1: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 1>), grid, block, 0, s, a); return launch_status();
-          case 2: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 2>), grid, block, 0, s, a); return launch_status();
-          case 3: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 3>), grid, block, 0, s, a); return launch_status();
-          case 7: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 7>), grid, block, 0, s, a); return launch_status();
-          case 15: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 15>), grid, block, 0, s, a); return launch_status();
-          case 16: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 16>), grid, block, 0, s, a); return launch_status();
-          case 8: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 8>), grid, block, 0, s, a); return launch_status();
-          case 4: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 4>), grid, block, 0, s, a); return launch_status();
-          case 32: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 32>), grid, block, 0, s, a); return launch_status();
-          case 39: hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, 39>), grid, block, 0, s, a); return launch_status();
-          default: break;
-        }
-      }
       hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16>), grid, block, 0, s, a);
       return launch_status();
     }

@@ -154,9 +154,13 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     r.end = (sg + 1 < a.n_kvseg) ? segs[sg + 1].start : Skv;
     r.step = segs[sg].ss * BKV;
   };
+  const bool one_seg = a.n_kvseg == 1;
   auto advance = [&](const SdpaSeg* segs, int ch, RowPtr& r) {
     const int64_t kj = r.row + BKV;
-    if (kj < r.end) {
+    if (one_seg) {  // uniform: rows past the end are never dereferenced
+      r.row = kj;
+      r.p += r.step;
+    } else if (kj < r.end) {
       r.row = kj;
       r.p += r.step;
     } else if (kj < Skv) {
