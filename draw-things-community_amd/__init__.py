@@ -31,6 +31,7 @@ ABI_SYMBOLS = (
     "dt_qx_bytes",
     "dt_depalettize_f16",
     "dt_dense_qx_f16",
+    "dt_dense_qx_heads_f16",
     "dt_qk_norm_rope_f16",
     "dt_sdpa_f16",
     "dt_sdpa_workspace_bytes",
@@ -50,6 +51,11 @@ class _QxWeight(ctypes.Structure):
 class _View4(ctypes.Structure):
     _fields_ = [("ptr", ctypes.c_void_p), ("stride_b", ctypes.c_int64), ("stride_s", ctypes.c_int64),
                 ("stride_h", ctypes.c_int64)]
+
+
+class _HeadEpilogue(ctypes.Structure):
+    _fields_ = [("gamma", ctypes.c_void_p), ("rot", ctypes.c_void_p), ("rot_pos0", ctypes.c_int64),
+                ("eps", ctypes.c_float), ("head_dim", ctypes.c_int32)]
 
 
 class _Segment(ctypes.Structure):
@@ -92,6 +98,10 @@ def lib():
         L.dt_dense_qx_f16.restype = i32
         L.dt_dense_qx_f16.argtypes = [vp, i64, i64, vp, i64, ctypes.POINTER(_QxWeight), i32,
                                       ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(i64), ctypes.c_uint32]
+        L.dt_dense_qx_heads_f16.restype = i32
+        L.dt_dense_qx_heads_f16.argtypes = [vp, i64, i64, vp, i64, ctypes.POINTER(_QxWeight), i32,
+                                            ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(i64),
+                                            ctypes.POINTER(_HeadEpilogue), ctypes.c_uint32]
         L.dt_qk_norm_rope_f16.restype = i32
         L.dt_qk_norm_rope_f16.argtypes = [vp, _View4, i32, i64, i32, i32, vp, f32, i32, vp, i64, f32]
         L.dt_sdpa_f16.restype = i32
@@ -250,9 +260,21 @@ class GEMMFlag:
     Float32 = 2
 
 
+@dataclass
+class HeadEpilogue:
+    """Per-head RMSNorm and RoPE fused behind a Dense: gamma [head_dim] or None, rot [>= rot_pos0 + M, head_dim] or None."""
+
+    gamma: "object" = None
+    rot: "object" = None
+    rot_pos0: int = 0
+    eps: float = 1e-6
+    head_dim: int = 128
+
+
 def dense_multi(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]], outs=None, flags: int = 0,
-                stream=None):
-    """Several Dense ops that share the input, one launch (x_q / x_k / x_v)."""
+                stream=None, epilogues: Optional[Sequence[Optional[HeadEpilogue]]] = None):
+    """Several Dense ops that share the input, one launch (x_q / x_k / x_v).  `epilogues[i]` (optional) fuses the
+    per-head RMSNorm / RoPE that follows projection i."""
     torch = _torch()
     _f16_cuda(x, "x")
     K = x.shape[-1]
@@ -271,8 +293,26 @@ def dense_multi(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object
     B = (vp * n)(*[None if b is None else _f16_cuda(b, "bias").data_ptr() for b in biases])
     Y = (vp * n)(*[o.data_ptr() for o in outs])
     LDY = (ctypes.c_int64 * n)(*[o.stride(0) for o in outs])
-    st = lib().dt_dense_qx_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, flags)
-    _check("dt_dense_qx_f16", st)
+    if epilogues is None:
+        st = lib().dt_dense_qx_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, flags)
+        _check("dt_dense_qx_f16", st)
+    else:
+        E = (_HeadEpilogue * n)()
+        for i, e in enumerate(epilogues):
+            if e is None:
+                E[i] = _HeadEpilogue(None, None, 0, 0.0, 128)
+                continue
+            if e.rot is not None:
+                _f16_cuda(e.rot, "rot")
+                if e.rot.dim() != 2 or e.rot.shape[1] != e.head_dim or not e.rot.is_contiguous() \
+                        or e.rot.shape[0] < e.rot_pos0 + M:
+                    raise ValueError("rot must be a contiguous [>= rot_pos0 + M, head_dim] table")
+            if e.gamma is not None and (_f16_cuda(e.gamma, "gamma").numel() != e.head_dim or not e.gamma.is_contiguous()):
+                raise ValueError("gamma must hold head_dim elements")
+            E[i] = _HeadEpilogue(None if e.gamma is None else e.gamma.data_ptr(),
+                                 None if e.rot is None else e.rot.data_ptr(), e.rot_pos0, e.eps, e.head_dim)
+        st = lib().dt_dense_qx_heads_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, E, flags)
+        _check("dt_dense_qx_heads_f16", st)
     lead = tuple(x.shape[:-1])
     return [o.reshape(lead + (o.shape[-1],)) if o.shape[0] == M and o.is_contiguous() else o for o in outs]
 

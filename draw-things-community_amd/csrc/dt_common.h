@@ -38,4 +38,30 @@ __device__ __forceinline__ uint16_t half_to_bits(half_t h) {
   return __builtin_bit_cast(uint16_t, h);
 }
 
+#if defined(__HIPCC__)
+// Combine the two half-waves (lanes l and l ^ 32 hold the same matrix column) without touching LDS:
+// v_permlane32_swap of a register with a copy of itself leaves {low, low} and {high, high}.
+__device__ __forceinline__ void halves32(float v, float& lo, float& hi) {
+  uint32_t a = __builtin_bit_cast(uint32_t, v), b = a;
+  asm volatile("" : "+v"(b));  // the swap needs two distinct registers
+  auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  uint32_t x0 = r[0], x1 = r[1];
+  // keeps the two results apart: without it the compiler has been seen to
+  // combine r[0] with itself when both inputs carry the same value
+  asm volatile("" : "+v"(x0), "+v"(x1));
+  lo = __builtin_bit_cast(float, x0);
+  hi = __builtin_bit_cast(float, x1);
+}
+__device__ __forceinline__ float max32(float v) {
+  float lo, hi;
+  halves32(v, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float sum32(float v) {
+  float lo, hi;
+  halves32(v, lo, hi);
+  return lo + hi;
+}
+#endif
+
 }  // namespace dt

@@ -12,6 +12,7 @@
 // K-tile and the unpack VALU/LDS work overlaps the matrix pipe.
 #include "dt_common.h"
 #include "dt_layout.h"
+#include "dt_qkprep.h"
 
 namespace dt {
 
@@ -34,6 +35,11 @@ struct DenseWeight {
   int64_t ldy;
   int32_t n;           // rows of this weight
   int32_t tile_begin;  // first N-tile index of this weight
+  // optional fused epilogue on 128-wide heads: RMSNorm weight, RoPE table, its first row, epsilon
+  const uint16_t* gamma;
+  const uint16_t* rot;
+  int64_t rot_pos0;
+  float eps;
 };
 
 struct DenseArgs {
@@ -103,16 +109,28 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const int lt = tid & 255;
   const int wn = wave & 1, wm = (wave >> 1) & 1 | ((wave >> 2) << 1);  // waves w and w+4 share a SIMD and take different m slices
 
-  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous
-  // run of tiles so the weight tiles it re-reads stay in that XCD's L2.
+  // Tile order: bands of 8 token tiles; inside a band feature tiles outermost,
+  // token tiles innermost.  Workgroups are dealt round-robin to the 8 XCDs;
+  // giving each XCD a contiguous run of that order makes the workgroups that
+  // run together on an XCD cover a compact 2-D block of tiles (8 x 4 at 32 CUs),
+  // so every X and W panel slice is fetched into that XCD's L2 once per block
+  // instead of once per tile column.
   const int total = a.tiles_m * a.tiles_n;
   int bid = blockIdx.x;
   {
     const int per = total / 8;
     if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
   }
-  const int tn = bid / a.tiles_m;
-  const int tm = bid - tn * a.tiles_m;
+  int tm, tn;
+  {
+    constexpr int GM = 8;
+    const int band_tiles = GM * a.tiles_n;
+    const int band = bid / band_tiles;
+    const int in_band = bid - band * band_tiles;
+    const int rows_in_band = (a.tiles_m - band * GM) < GM ? (a.tiles_m - band * GM) : GM;
+    tn = in_band / rows_in_band;
+    tm = band * GM + (in_band - tn * rows_in_band);
+  }
 
   int wi = 0;
 #pragma unroll
@@ -389,6 +407,97 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   if (t < nk) iteration(t, R2, R1);
   if (t + 1 < nk) iteration(t + 1, R0, R2);
 
+  // ---- fused epilogue: per-head RMSNorm and RoPE on the way out ---------------
+  // A wave's 128 features are exactly one head, and every lane pair (l, l ^ 32)
+  // holds all 128 of them for its token, adjacent (re, im) pairs in one lane:
+  // the norm's reduction and the rotation need no data movement.  Rounds to
+  // fp16 after the Dense, after the norm and after the rotation, as the
+  // op-by-op graph does.
+  if constexpr (WN == 128) {
+    if (w.gamma || w.rot) {
+      const int nh = n0 + wn * WN;  // first feature of this wave's head
+      if (nh >= w.n) return;        // heads are whole: this wave's slice lies past the last one
+#pragma unroll
+      for (int j = 0; j < TM; j++) {
+        const int gm = m0 + wm * WM + j * 32 + l32;
+        const int gmc = gm < a.m ? gm : a.m - 1;
+        uint16_t* yrow = w.y + (int64_t)gmc * w.ldy;
+        float y[TN][16];
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            const int nl = i * 32 + 8 * g + 4 * hi;
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (w.bias) {
+              const uint2_t bb = *reinterpret_cast<const uint2_t*>(w.bias + nh + nl);
+              bv[0] = (float)bits_to_half((uint16_t)bb[0]);
+              bv[1] = (float)bits_to_half((uint16_t)(bb[0] >> 16));
+              bv[2] = (float)bits_to_half((uint16_t)bb[1]);
+              bv[3] = (float)bits_to_half((uint16_t)(bb[1] >> 16));
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const float v = (float)(half_t)(acc[i][j][4 * g + e] + bv[e]);
+              y[i][4 * g + e] = v;
+              ss += v * v;
+            }
+          }
+        if (w.gamma) {
+          const float inv = 1.0f / sqrtf(sum32(ss) / (float)WN + w.eps);
+#pragma unroll
+          for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+              const uint2_t gg = *reinterpret_cast<const uint2_t*>(w.gamma + i * 32 + 8 * g + 4 * hi);
+              const float gv[4] = {(float)bits_to_half((uint16_t)gg[0]), (float)bits_to_half((uint16_t)(gg[0] >> 16)),
+                                   (float)bits_to_half((uint16_t)gg[1]), (float)bits_to_half((uint16_t)(gg[1] >> 16))};
+#pragma unroll
+              for (int e = 0; e < 4; e++) y[i][4 * g + e] = (float)(half_t)(y[i][4 * g + e] * inv * gv[e]);
+            }
+        }
+        if (w.rot) {
+          const uint16_t* rrow = w.rot + (w.rot_pos0 + gmc) * WN;
+#pragma unroll
+          for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+              const uint2_t rr = *reinterpret_cast<const uint2_t*>(rrow + i * 32 + 8 * g + 4 * hi);
+#pragma unroll
+              for (int pr = 0; pr < 2; pr++) {
+                const float c = (float)bits_to_half((uint16_t)rr[pr]), sn = (float)bits_to_half((uint16_t)(rr[pr] >> 16));
+                const float re = y[i][4 * g + 2 * pr], im = y[i][4 * g + 2 * pr + 1];
+                y[i][4 * g + 2 * pr] = (float)(half_t)(re * c - im * sn);
+                y[i][4 * g + 2 * pr + 1] = (float)(half_t)(re * sn + im * c);
+              }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+          uint32_t pk[4][2];
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            pk[g][0] = pack_h2(y[i][4 * g], y[i][4 * g + 1]);
+            pk[g][1] = pack_h2(y[i][4 * g + 2], y[i][4 * g + 3]);
+          }
+#pragma unroll
+          for (int gp = 0; gp < 2; gp++) {
+            uint32_t run[4];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+              auto r = __builtin_amdgcn_permlane32_swap(pk[2 * gp][e], pk[2 * gp + 1][e], false, false);
+              run[e] = r[0];
+              run[2 + e] = r[1];
+            }
+            if (gm < a.m) *reinterpret_cast<uint4_t*>(yrow + nh + i * 32 + 16 * gp + 8 * hi) = uint4_t{run[0], run[1], run[2], run[3]};
+          }
+        }
+      }
+      return;
+    }
+  }
+
   // ---- epilogue: bias, round once to fp16, 16-byte stores -------------------
   // Accumulator block (i, j): lane holds token column (lane & 31) and features
   // 8 * g + 4 * (lane / 32) + (0..3) for g = 0..3.  Swapping the odd groups of
@@ -528,8 +637,25 @@ static int choose_pal_mode(int qbits, int nib, int64_t K, int BN) {
 DT_EXPORT dt_status dt_dense_qx_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,
                                     const dt_qx_weight* W, int32_t n_weights, const uint16_t* const* bias,
                                     uint16_t* const* Y, const int64_t* ldy, uint32_t flags) {
+  return dt_dense_qx_heads_f16(stream, M, K, X, ldx, W, n_weights, bias, Y, ldy, nullptr, flags);
+}
+
+DT_EXPORT dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,
+                                          const dt_qx_weight* W, int32_t n_weights, const uint16_t* const* bias,
+                                          uint16_t* const* Y, const int64_t* ldy, const dt_head_epilogue* epi,
+                                          uint32_t flags) {
   using namespace dt;
   (void)flags;
+  if (epi && n_weights > 0) {
+    for (int i = 0; i < n_weights; i++) {
+      if (!epi[i].gamma && !epi[i].rot) continue;
+      if (epi[i].head_dim <= 0 || epi[i].head_dim % 2 != 0 || epi[i].head_dim > 128) return DT_NO_KERNEL;
+      if (epi[i].rot && epi[i].rot_pos0 < 0) return DT_INVALID;
+      if (Y && ldy && M > 0 && ((ldy[i] & 1) || (reinterpret_cast<uintptr_t>(Y[i]) & 3))) return DT_INVALID;
+      if (epi[i].rot && (reinterpret_cast<uintptr_t>(epi[i].rot) & 3)) return DT_INVALID;
+      if (W && K > 0 && W[i].count >= 0 && (W[i].count / K) % epi[i].head_dim != 0) return DT_INVALID;
+    }
+  }
   if (M < 0 || K <= 0 || n_weights <= 0 || !W || !Y || !ldy) return DT_INVALID;
   if (M > 0x7fffffff || K > 0x7fffffff) return DT_INVALID;
   for (int i = 0; i < n_weights; i++) {
@@ -553,6 +679,34 @@ DT_EXPORT dt_status dt_dense_qx_f16(dt_stream stream, int64_t M, int64_t K, cons
     const int64_t n_rows0 = w0.count / K;
     bool tiled = x_ok && n_rows0 > 0 && (reinterpret_cast<uintptr_t>(w0.data) & 15) == 0 &&
                  (w0.qbits == 16 || w0.nib % 32 == 0);
+    // fused head epilogue: in the tiled kernel for 128-wide heads that start on a 16-byte aligned,
+    // 8-element-strided output; otherwise the Dense runs plain and the norm / rotation pass follows
+    auto wants_epi = [&](int wi) { return epi && (epi[wi].gamma || epi[wi].rot); };
+    auto fusable = [&](int wi) {
+      return epi[wi].head_dim == 128 && (ldy[wi] % 8 == 0) && ((reinterpret_cast<uintptr_t>(Y[wi]) & 15) == 0) &&
+             (!epi[wi].gamma || (reinterpret_cast<uintptr_t>(epi[wi].gamma) & 7) == 0) &&
+             (!epi[wi].rot || (reinterpret_cast<uintptr_t>(epi[wi].rot) & 7) == 0) &&
+             (!bias || !bias[wi] || (reinterpret_cast<uintptr_t>(bias[wi]) & 7) == 0);
+    };
+    auto epilogue_pass = [&](int wi) -> dt_status {
+      QkPrepArgs p;
+      p.src = Y[wi];
+      p.dst = Y[wi];
+      p.src_sb = p.dst_sb = 0;
+      p.src_ss = p.dst_ss = ldy[wi];
+      p.src_sh = p.dst_sh = epi[wi].head_dim;
+      p.B = 1;
+      p.S = M;
+      p.H = (int32_t)((W[wi].count / K) / epi[wi].head_dim);
+      p.D = epi[wi].head_dim;
+      p.gamma = epi[wi].gamma;
+      p.eps = epi[wi].eps;
+      p.norm_per_head = 1;
+      p.rot = epi[wi].rot;
+      p.rot_pos0 = epi[wi].rot_pos0;
+      p.post_scale = 1.0f;
+      return qk_prep_launch(s, p);
+    };
     if (!tiled) {
       if (n_rows0 > 0) {
         int64_t outs = M * n_rows0;
@@ -562,13 +716,21 @@ DT_EXPORT dt_status dt_dense_qx_f16(dt_stream stream, int64_t M, int64_t K, cons
                            bias ? bias[i] : nullptr, Y[i], ldy[i]);
         dt_status st = launch_status();
         if (st != DT_OK) return st;
+        if (wants_epi(i)) {
+          st = epilogue_pass(i);
+          if (st != DT_OK) return st;
+        }
       }
       i++;
       continue;
     }
     // tile shape: big tiles when there is enough work to fill 256 CUs with them
-    const bool big = (M >= 1024) && (n_rows0 >= 256);
-    const int BM = big ? 256 : 128, BN = big ? 256 : 128;
+    bool any_fused = false;
+    for (int j = i; j < n_weights && j < i + kMaxWeights; j++) any_fused = any_fused || (wants_epi(j) && fusable(j));
+    const bool big = ((M >= 1024) && (n_rows0 >= 256)) || any_fused;  // the fused epilogue needs the 128-feature wave slice
+    // few token rows: halve the token tile so that more workgroups share the work
+    const bool narrow = big && M < 1024;
+    const int BM = big ? (narrow ? 128 : 256) : 128, BN = big ? 256 : 128;
     DenseArgs a;
     a.x = X;
     a.ldx = ldx;
@@ -577,6 +739,7 @@ DT_EXPORT dt_status dt_dense_qx_f16(dt_stream stream, int64_t M, int64_t K, cons
     a.nib = w0.qbits == 16 ? 32 : w0.nib;
     a.tiles_m = (int)((M + BM - 1) / BM);
     int tiles_n = 0, cnt = 0;
+    const int first = i;
     while (i < n_weights && cnt < kMaxWeights) {
       const dt_qx_weight& w = W[i];
       const int64_t n_rows = w.count / K;
@@ -589,6 +752,11 @@ DT_EXPORT dt_status dt_dense_qx_f16(dt_stream stream, int64_t M, int64_t K, cons
       a.w[cnt].ldy = ldy[i];
       a.w[cnt].n = (int32_t)n_rows;
       a.w[cnt].tile_begin = tiles_n;
+      const bool fuse = big && wants_epi(i) && fusable(i);
+      a.w[cnt].gamma = fuse ? epi[i].gamma : nullptr;
+      a.w[cnt].rot = fuse ? epi[i].rot : nullptr;
+      a.w[cnt].rot_pos0 = fuse ? epi[i].rot_pos0 : 0;
+      a.w[cnt].eps = fuse ? epi[i].eps : 0.f;
       tiles_n += (int)((n_rows + BN - 1) / BN);
       cnt++;
       i++;
@@ -598,8 +766,15 @@ DT_EXPORT dt_status dt_dense_qx_f16(dt_stream stream, int64_t M, int64_t K, cons
     a.tiles_n = tiles_n;
     if ((int64_t)a.tiles_m * tiles_n > 0x7fffffff) return DT_NO_KERNEL;
     const int mode = choose_pal_mode(w0.qbits, a.nib, K, BN);
-    dt_status st = big ? launch_tiled_q<256, 256>(s, a, w0.qbits, mode) : launch_tiled_q<128, 128>(s, a, w0.qbits, mode);
+    dt_status st = !big ? launch_tiled_q<128, 128>(s, a, w0.qbits, mode)
+                   : narrow ? launch_tiled_q<128, 256>(s, a, w0.qbits, mode)
+                            : launch_tiled_q<256, 256>(s, a, w0.qbits, mode);
     if (st != DT_OK) return st;
+    for (int j = first; j < i; j++)
+      if (wants_epi(j) && !(big && fusable(j))) {
+        st = epilogue_pass(j);
+        if (st != DT_OK) return st;
+      }
   }
   return DT_OK;
 }

@@ -28,30 +28,6 @@ constexpr int QROWS = QWAVES * 32;
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-// Combine the two half-waves (lanes l and l ^ 32 hold the same query) without touching LDS:
-// v_permlane32_swap of a register with a copy of itself leaves {low, low} and {high, high}.
-__device__ __forceinline__ void halves32(float v, float& lo, float& hi) {
-  uint32_t a = __builtin_bit_cast(uint32_t, v), b = a;
-  asm volatile("" : "+v"(b));  // the swap needs two distinct registers
-  auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
-  uint32_t x0 = r[0], x1 = r[1];
-  // keeps the two results apart: without it the compiler has been seen to
-  // combine r[0] with itself when both inputs carry the same value
-  asm volatile("" : "+v"(x0), "+v"(x1));
-  lo = __builtin_bit_cast(float, x0);
-  hi = __builtin_bit_cast(float, x1);
-}
-__device__ __forceinline__ float max32(float v) {
-  float lo, hi;
-  halves32(v, lo, hi);
-  return fmaxf(lo, hi);
-}
-__device__ __forceinline__ float sum32(float v) {
-  float lo, hi;
-  halves32(v, lo, hi);
-  return lo + hi;
-}
-
 // LDS layouts (measured bank-conflict free on this part: 64 banks, 16 lanes of
 // a 16-byte access or 32 lanes of an 8-byte access per clock).
 // K tile: [64 keys][DP] halfs; 16-byte chunk c of key row r is stored at a

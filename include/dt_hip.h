@@ -120,6 +120,36 @@ dt_status dt_dense_qx_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t
                           uint16_t* const* Y, const int64_t* ldy, uint32_t flags);
 
 /*
+ * Dense with the per-head RMSNorm and the RoPE rotation that follow it in the
+ * attention blocks fused into the GEMM epilogue (Dense -> reshaped([b, s, h, k])
+ * -> RMSNorm(axis: [3]) -> cmul(rot), Models/Flux1.swift:174-188): Q and K leave
+ * the projection already normalised and rotated, with no extra pass over them.
+ * epi: HOST array of n_weights entries, or NULL (then identical to
+ * dt_dense_qx_f16).  An entry with gamma == NULL and rot == NULL leaves that
+ * weight's output plain (x_v).  Each output row is treated as heads of
+ * `head_dim` features; rounding happens after the Dense, after the norm and
+ * after the rotation, exactly as the three separate ops round.
+ *   gamma    : RMSNorm weight [head_dim] (x_norm_q / x_norm_k), or NULL
+ *   eps      : RMSNorm epsilon
+ *   rot      : [>= rot_pos0 + M, head_dim] fp16 table of interleaved (cos, sin), or NULL
+ *   rot_pos0 : table row of X's first row (offset of this stream in the joint sequence)
+ *   head_dim : 128 runs inside the GEMM epilogue; other even values <= 128 run
+ *              as a separate pass after the GEMM (same results)
+ */
+typedef struct {
+  const uint16_t* gamma;
+  const uint16_t* rot;
+  int64_t rot_pos0;
+  float eps;
+  int32_t head_dim;
+} dt_head_epilogue;
+
+dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,
+                                const dt_qx_weight* W, int32_t n_weights, const uint16_t* const* bias,
+                                uint16_t* const* Y, const int64_t* ldy, const dt_head_epilogue* epi,
+                                uint32_t flags);
+
+/*
  * In place on a [B, S, H, D] view: optional RMSNorm, then optional RoPE.
  *   gamma       : RMSNorm weight, [D] when norm_per_head != 0 (Flux:
  *                 RMSNorm(axis: [3]), Models/Flux1.swift:165), [H*D] when 0

@@ -201,3 +201,49 @@ def test_dense_flux_qkv_full_size_sampled(dthip, oracle, torch_cuda):
         normal = a.abs() >= 2.0 ** -13
         assert torch.equal((a * 2)[normal], b[normal])
         assert float((a.float() * 2 - b.float()).abs().max()) <= 2.0 ** -23
+
+
+@pytest.mark.parametrize("M,head_dim,q,nib", [(700, 128, 6, 4096), (300, 128, 8, 16384), (130, 64, 6, 4096)])
+def test_dense_fused_head_norm_rope(dthip, oracle, torch_cuda, M, head_dim, q, nib):
+    """x_q / x_k / x_v with the per-head RMSNorm + RoPE of Q and K fused behind the projection (V left plain):
+    equals Dense -> RMSNorm(axis: [3]) -> cmul(rot) of the oracle.  head_dim 128 runs inside the GEMM epilogue,
+    64 as a pass after it."""
+    torch = torch_cuda
+    rng = np.random.default_rng(M + head_dim)
+    K, H = 512, 3
+    N = H * head_dim
+    pos0 = 11
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    ws, packs, biases, gammas = [], [], [], []
+    for i in range(3):
+        w, p = make_weight(dthip, oracle, rng, N, K, q, nib, std=0.05)
+        ws.append(w)
+        packs.append(p)
+        biases.append((rng.standard_normal(N) * 0.05).astype(np.float16))
+        gammas.append((1 + 0.05 * rng.standard_normal(head_dim)).astype(np.float16))
+    theta = rng.uniform(-3, 3, size=(pos0 + M, head_dim // 2))
+    rot = np.empty((pos0 + M, head_dim), np.float16)
+    rot[:, 0::2] = np.cos(theta)
+    rot[:, 1::2] = np.sin(theta)
+    rot_d = to_dev(torch, rot)
+    epi = [dthip.HeadEpilogue(to_dev(torch, gammas[0]), rot_d, pos0, 1e-6, head_dim),
+           dthip.HeadEpilogue(to_dev(torch, gammas[1]), rot_d, pos0, 1e-6, head_dim), None]
+    out = torch.zeros((M, 3 * N), dtype=torch.float16, device="cuda")
+    outs = [out[:, i * N:(i + 1) * N] for i in range(3)]
+    print("dense fused heads", M, head_dim, q, flush=True)
+    dthip.dense_multi(to_dev(torch, X), ws, [to_dev(torch, b) for b in biases], outs=outs, epilogues=epi)
+    got = out.cpu().numpy()
+    for i in range(3):
+        y = oracle.C.dense_qx(X, packs[i], q, nib, N, biases[i])
+        if i < 2:
+            y = oracle.C.cmul(oracle.C.rmsnorm(y.reshape(M, H, head_dim), gammas[i], 1e-6), rot[pos0:]).reshape(M, N)
+        mx, rr = oracle.err_stats(got[:, i * N:(i + 1) * N], y)
+        assert mx <= MAX_ABS and rr <= 2 * REL_RMS, (i, mx, rr)
+    # norm only / rotation only
+    for epi1 in (dthip.HeadEpilogue(to_dev(torch, gammas[0]), None, 0, 1e-6, head_dim),
+                 dthip.HeadEpilogue(None, rot_d, pos0, 1e-6, head_dim)):
+        o1 = dthip.dense_multi(to_dev(torch, X), [ws[0]], [None], epilogues=[epi1])[0].cpu().numpy()
+        y = oracle.C.dense_qx(X, packs[0], q, nib, N, None).reshape(M, H, head_dim)
+        y = oracle.C.rmsnorm(y, gammas[0], 1e-6) if epi1.rot is None else oracle.C.cmul(y, rot[pos0:])
+        mx, rr = oracle.err_stats(o1, y.reshape(M, N))
+        assert mx <= MAX_ABS and rr <= 2 * REL_RMS, (mx, rr)
