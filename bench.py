@@ -20,6 +20,9 @@ if ROOT not in sys.path:
 
 PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
+# counters read for a 256 MiB device copy (x2.00 and x1.00); the summary is profiles/bench_flux_block_counters.txt
+MEASURED_TRAFFIC_BYTES = {"dense_qkv_image": 1.073e9, "sdpa": 1.327e8}
 
 
 def main():
@@ -187,13 +190,19 @@ def main():
     # dominant kernel of the step (by time): roofline against the fp16 MFMA peak
     dense_ms = ms["dense_qkv_image_M4096"] + ms["dense_qkv_text_M512"] + ms["dense_out_2x"]
     if ms["sdpa_S4608"] >= ms["dense_qkv_image_M4096"]:
-        dom, dom_flop, dom_ms = "sdpa_kernel<128,2> S=4608 H=24", flop_sdpa, ms["sdpa_S4608"]
+        dom, dom_flop, dom_ms, dom_tr = "sdpa_kernel<128> S=4608 H=24", flop_sdpa, ms["sdpa_S4608"], "sdpa"
     else:
-        dom, dom_flop, dom_ms = "dense_qx_kernel<6,256,256> M=4096 N=3x3072 K=3072", 2.0 * HW * C * 3 * C, ms["dense_qkv_image_M4096"]
+        dom, dom_flop, dom_ms, dom_tr = ("dense_qx_kernel<6,256,256> M=4096 N=3x3072 K=3072 (fused norm/RoPE epilogue)",
+                                          2.0 * HW * C * 3 * C, ms["dense_qkv_image_M4096"], "dense_qkv_image")
     roofline = {
         "kernel": dom, "bound": "mfma", "achieved": round(tf(dom_flop, dom_ms), 2), "peak": PEAK_F16_TFLOPS,
-        "unit": "TFLOP/s", "frac": round(tf(dom_flop, dom_ms) / PEAK_F16_TFLOPS, 4), "traffic": None,
-        "flop_per_launch": dom_flop, "avg_launch_ms": round(dom_ms, 4),
+        "unit": "TFLOP/s", "frac": round(tf(dom_flop, dom_ms) / PEAK_F16_TFLOPS, 4),
+        "traffic": MEASURED_TRAFFIC_BYTES[dom_tr], "flop_per_launch": dom_flop, "avg_launch_ms": round(dom_ms, 4),
+        "others": {
+            "sdpa_kernel<128> S=4608 H=24": {"achieved": round(tf(flop_sdpa, ms["sdpa_S4608"]), 2),
+                                             "frac": round(tf(flop_sdpa, ms["sdpa_S4608"]) / PEAK_F16_TFLOPS, 4),
+                                             "traffic": MEASURED_TRAFFIC_BYTES["sdpa"]},
+        },
     }
 
     # ---------------- CPU baseline: the oracle on a bounded sample ----------------
