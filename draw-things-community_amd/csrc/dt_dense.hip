@@ -74,6 +74,20 @@ struct RowCursor {
 // the operand reads, the 4-lanes-per-row tile writes and the row-per-lane writes.
 __device__ __forceinline__ int lds_chunk(int row, int c) { return row * BK + ((c ^ ((row >> 2) & 3)) << 3); }
 
+// Pair slots are [rows][64 halfs] (two K-tiles side by side): logical chunk c
+// (0..7) of row r sits at 16-byte slot c ^ (r / 2 % 8), which puts 16
+// consecutive rows of one chunk column on 16 distinct 16-byte bank groups.
+__device__ __forceinline__ int pair_chunk(int row, int slot) { return slot ^ ((row >> 1) & 7); }
+
+constexpr int kWaitVm0 = 0x0f70;  // s_waitcnt vmcnt(0), other counters untouched
+
+// One wave-wide memory -> LDS transfer: lane l's 16 bytes at g land at LDS
+// address lds + 16 * l (lds wave-uniform).
+__device__ __forceinline__ void load_to_lds_16(const void* g, half_t* lds) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                   (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+}
+
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
   return (uint32_t)half_to_bits((half_t)a) | ((uint32_t)half_to_bits((half_t)b) << 16);
 }
@@ -91,15 +105,23 @@ template <int Q, int BM, int BN, int MODE>
 __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   constexpr int WN = BN / 2, WM = BM / 4;   // per-wave slice: WN features x WM tokens
   constexpr int TN = WN / 32, TM = WM / 32;
-  constexpr int A_CHUNKS = BM * (BK / 8) / 512;  // 16-byte chunks of X per thread per K-tile
-  constexpr int B_CHUNKS = BN * (BK / 8) / 512;  // plain fp16 weight: 16-byte chunks per thread
+  constexpr int AP = BM * (BK / 4) / 512;  // 16-byte chunks of X per thread per pair of K-tiles
+  constexpr int BP = MODE == kPlainF16 ? BN * (BK / 4) / 512 : 0;  // plain fp16 weight: the same
   constexpr int QW = MODE == kPlainF16 ? 1 : Q;  // dwords per granule
-  constexpr int NST = 3;                         // LDS ring depth
-  constexpr int A_STAGE = BM * BK, B_STAGE = BN * BK;
-  static_assert(BM % 128 == 0 && BN % 64 == 0 && BN <= 256, "tile");
+  constexpr int HW = (QW + 1) / 2;               // dwords that hold either half of a granule
+  constexpr int NST = 3;                         // ring depth of the unpacked weight tiles
+  constexpr int B_STAGE = BN * BK;
+  constexpr int PROW = 2 * BK;                   // halfs per row of a pair slot
+  static_assert(BM % 128 == 0 && BN % 128 == 0 && BN <= 256, "tile");
 
-  __shared__ __attribute__((aligned(16))) half_t As[NST * A_STAGE];
-  __shared__ __attribute__((aligned(16))) half_t Bs[NST * B_STAGE];
+  // X (and a plain fp16 W) lives in two pair slots, each holding two K-tiles
+  // as [rows][64 halfs]; the slots are separate arrays so that reads of one
+  // are known not to touch the other while a load into it is in flight.
+  __shared__ __attribute__((aligned(1024))) half_t XsA[BM * PROW];
+  __shared__ __attribute__((aligned(1024))) half_t XsB[BM * PROW];
+  __shared__ __attribute__((aligned(1024))) half_t WpA[MODE == kPlainF16 ? BN * PROW : 8];
+  __shared__ __attribute__((aligned(1024))) half_t WpB[MODE == kPlainF16 ? BN * PROW : 8];
+  __shared__ __attribute__((aligned(16))) half_t Bs[MODE == kPlainF16 ? 8 : NST * B_STAGE];
   __shared__ __attribute__((aligned(16))) uint16_t Pal[(MODE == kPalShared || MODE == kPalRow) ? kPalLdsBytes / 2 : 8];
 
   const int tid = threadIdx.x;
@@ -143,61 +165,51 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const int nk = K / BK;
   const QxLayout lay = make_layout(Q, a.nib);
   const uint32_t pal_bytes = (uint32_t)lay.pal_bytes;
-  // Rows of X (and of a plain fp16 W) are K * 2 bytes apart, a stride that maps
-  // a K-tile's 64-byte row segments onto very few memory channels.  Each
-  // workgroup walks the K-tiles in a rotated order so that concurrent
-  // workgroups pull from different channels.
-  const int rot = (int)(((unsigned)tm * 5u + (unsigned)tn * 11u) % (unsigned)nk);
-
   // ---- per-thread load coordinates (32-bit byte offsets from uniform bases) ----
-  uint32_t a_off[A_CHUNKS];
-  int a_dst[A_CHUNKS];
+  // X (and a plain fp16 W) goes from memory straight into LDS, two K-tiles at
+  // a time: eight lanes cover one row's 128 contiguous bytes, so every cache
+  // line is requested once, whole.  A wave's load instruction fills 1 KB of
+  // LDS = 8 rows of a pair slot, lane l landing on 16-byte slot l % 8 of row
+  // l / 8; the lane fetches the chunk that the swizzle assigns to that slot.
+  uint32_t a_off[AP];
 #pragma unroll
-  for (int i = 0; i < A_CHUNKS; i++) {
-    int c = tid + i * 512;
-    int row = c >> 2, kc = c & 3;
+  for (int i = 0; i < AP; i++) {
+    const int row = 8 * (wave * AP + i) + (lane >> 3);
+    const int c8 = pair_chunk(row, lane & 7);
     int gm = m0 + row;
     if (gm >= a.m) gm = a.m - 1;
-    a_off[i] = (uint32_t)(((int64_t)gm * a.ldx + kc * 8) * 2);
-    a_dst[i] = lds_chunk(row, kc);
+    a_off[i] = (uint32_t)(((int64_t)gm * a.ldx + c8 * 8) * 2);
   }
   const char* xbase = reinterpret_cast<const char*>(a.x);
   const char* wbase = reinterpret_cast<const char*>(w.data);
 
-  // weight row of this thread (both threads of a pair read the row's granule, each unpacks one half)
+  // weight row of this thread (two threads per row; each loads and unpacks one half of the row's granule)
   const bool b_active = (BN >= 256) || (lt < BN);
   const int b_row = lt < BN ? lt : BN - 1;
-  RowCursor cur, cur0;  // current tile, and tile 0 for the wrap-around
+  RowCursor cur;
   int64_t pal_first_block = 0;
   if constexpr (MODE == kPalShared) pal_first_block = ((int64_t)n0 * K) / a.nib;
   if constexpr (MODE != kPlainF16) {
     int gn = n0 + b_row;
     if (gn >= w.n) gn = w.n - 1;
-    auto cursor_at = [&](int tile) {
-      const int64_t e = (int64_t)gn * K + (int64_t)tile * BK;
-      const int64_t blk = e / a.nib;
-      const int64_t r = e - blk * a.nib;
-      RowCursor c;
-      c.off = (uint32_t)index_byte_offset(lay, blk, r);
-      c.poff = (uint32_t)palette_offset(lay, blk);
-      c.r = (int32_t)r;
-      c.slot = MODE == kPalShared ? (int32_t)(blk - pal_first_block) : b_row;
-      return c;
-    };
-    cur = cursor_at(rot);
-    cur0 = cursor_at(0);
+    const int64_t e = (int64_t)gn * K;
+    const int64_t blk = e / a.nib;
+    const int64_t r = e - blk * a.nib;
+    cur.off = (uint32_t)index_byte_offset(lay, blk, r);
+    cur.poff = (uint32_t)palette_offset(lay, blk);
+    cur.r = (int32_t)r;
+    cur.slot = MODE == kPalShared ? (int32_t)(blk - pal_first_block) : b_row;
+    if (second) cur.off += 4 * (Q / 2);  // first dword that holds an index of the granule's second half
   }
-  uint32_t bf_off[B_CHUNKS > 0 ? B_CHUNKS : 1];
-  int bf_dst[B_CHUNKS > 0 ? B_CHUNKS : 1];
+  uint32_t bf_off[BP > 0 ? BP : 1];
   if constexpr (MODE == kPlainF16) {
 #pragma unroll
-    for (int i = 0; i < B_CHUNKS; i++) {
-      int c = tid + i * 512;
-      int row = c >> 2, kc = c & 3;
+    for (int i = 0; i < BP; i++) {
+      const int row = 8 * (wave * BP + i) + (lane >> 3);
+      const int c8 = pair_chunk(row, lane & 7);
       int gn = n0 + row;
       if (gn >= w.n) gn = w.n - 1;
-      bf_off[i] = (uint32_t)(((int64_t)gn * K + kc * 8) * 2);
-      bf_dst[i] = lds_chunk(row, kc);
+      bf_off[i] = (uint32_t)(((int64_t)gn * K + c8 * 8) * 2);
     }
   }
 
@@ -228,45 +240,47 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       reinterpret_cast<uint32_t*>(Pal)[i] = src[e];
     }
   };
-  if constexpr (MODE == kPalRow) load_row_palettes(rot * BK);
+  if constexpr (MODE == kPalRow) load_row_palettes(0);
 
-  // ---- register staging: two sets so a tile's loads fly for a whole iteration ----
-  struct RegSet {
-    uint4_t x[A_CHUNKS];
-    uint4_t wf[B_CHUNKS > 0 ? B_CHUNKS : 1];  // plain fp16 weight chunks
-    uint32_t b[QW];                           // packed indices of the row's granule
+  // ---- staging --------------------------------------------------------------
+  struct IdxSet {
+    uint32_t b[HW];  // the dwords that hold this thread's half of the row's granule
     uint32_t poff;
     int32_t slot;
   };
-  RegSet R0, R1, R2;
+  IdxSet WS[2];  // tile T travels in WS[T % 2]
+  const int last_pair = nk / 2 - 1;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
 
-  // Loads the tile the cursor points at (the last tile is re-read harmlessly by
-  // the final iterations) and moves the cursor on by one tile.
-  int next_tile = rot;  // K-tile the cursor points at
-  int issued = 0;       // tiles loaded so far
-  auto issue_loads = [&](RegSet& R) {
-    const int k0 = next_tile * BK;
-    const char* xk = xbase + (int64_t)k0 * 2;
+  // Starts the memory -> LDS transfer of K-tile pair q into a pair slot (pairs
+  // past the end re-read the last one, harmlessly).
+  auto issue_pair = [&](half_t* xs, half_t* wp, int q) {
+    if (q > last_pair) q = last_pair;
+    const int64_t kb = (int64_t)q * (4 * BK);  // byte offset of the pair inside a row
+    const char* xk = xbase + kb;
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; i++) R.x[i] = ld_global_16(xk + a_off[i]);
+    for (int i = 0; i < AP; i++)
+      load_to_lds_16(xk + a_off[i], xs + (wave_u * AP + i) * 512);
     if constexpr (MODE == kPlainF16) {
-      const char* wk = wbase + (int64_t)k0 * 2;
+      const char* wk = wbase + kb;
 #pragma unroll
-      for (int i = 0; i < B_CHUNKS; i++) R.wf[i] = ld_global_16(wk + bf_off[i]);
-    } else {
+      for (int i = 0; i < BP; i++)
+        load_to_lds_16(wk + bf_off[i], wp + (wave_u * BP + i) * 512);
+    }
+  };
+
+  // Loads the indices of the tile the cursor points at (the last tile is re-read
+  // harmlessly by the final iterations) and moves the cursor on by one tile.
+  int issued = 0;  // tiles loaded so far
+  auto issue_idx = [&](IdxSet& R) {
+    if constexpr (MODE != kPlainF16) {
       const uint32_t* src = reinterpret_cast<const uint32_t*>(wbase + cur.off);
 #pragma unroll
-      for (int i = 0; i < QW; i++) R.b[i] = src[i];
+      for (int i = 0; i < HW; i++) R.b[i] = src[i];
       R.poff = cur.poff;
       R.slot = cur.slot;
-    }
-    if (issued + 1 < nk) {
-      issued++;
-      next_tile++;
-      if (next_tile == nk) {
-        next_tile = 0;
-        if constexpr (MODE != kPlainF16) cur = cur0;
-      } else if constexpr (MODE != kPlainF16) {
+      if (issued + 1 < nk) {
+        issued++;
         cur.r += BK;
         cur.off += 4 * Q;
         if (cur.r >= a.nib) {
@@ -279,21 +293,30 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     }
   };
 
-  auto stage_to_lds = [&](const RegSet& R, int stage) {
-    half_t* Asd = As + stage * A_STAGE;
-    half_t* Bsd = Bs + stage * B_STAGE;
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; i++) *reinterpret_cast<uint4_t*>(&Asd[a_dst[i]]) = R.x[i];
-    if constexpr (MODE == kPlainF16) {
-#pragma unroll
-      for (int i = 0; i < B_CHUNKS; i++) *reinterpret_cast<uint4_t*>(&Bsd[bf_dst[i]]) = R.wf[i];
-    } else {
+  // Unpacks the granule held in R, looks it up and writes the weights into a ring stage.
+  auto stage_to_lds = [&](const IdxSet& R, int stage) {
+    if constexpr (MODE != kPlainF16) {
+      half_t* Bsd = Bs + stage * B_STAGE;
       if (b_active) {
         uint32_t idx[16];
-        if (second)
-          unpack16<Q, 1>(R.b, idx);
-        else
-          unpack16<Q, 0>(R.b, idx);
+        uint32_t mine[HW];
+#pragma unroll
+        for (int j = 0; j < HW; j++) {
+          mine[j] = R.b[j];
+          // Pins the unpacking to this point: hoisted above the preceding barrier
+          // it would drag the wait for the index load along with it.
+          asm volatile("" : "+v"(mine[j]));
+        }
+        uint32_t g[QW];  // the granule with only this thread's dwords filled in
+        if (second) {
+#pragma unroll
+          for (int j = 0; j < QW; j++) g[j] = (j >= Q / 2 && j - Q / 2 < HW) ? mine[j - Q / 2] : 0u;
+          unpack16<Q, 1>(g, idx);
+        } else {
+#pragma unroll
+          for (int j = 0; j < QW; j++) g[j] = j < HW ? mine[j] : 0u;
+          unpack16<Q, 0>(g, idx);
+        }
         uint32_t o[8];
         const uint16_t* pal;
         if constexpr (MODE == kPalGlobal)
@@ -320,17 +343,29 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // ---- fragment double buffer --------------------------------------------
   // MFMA A operand = W rows (features), B operand = X rows (tokens); lane holds
   // row (lane & 31), k-slots 8 * (lane / 32) .. + 7 of the 16-wide k-step.
+  // In a pair slot the 16-byte chunk c (0..7: tile parity * 4 + k-step * 2 +
+  // half) of row r sits at slot c ^ (r / 2 % 8); rows 32 apart share a swizzle.
   const int l32 = lane & 31, hi = lane >> 5;
+  const int xrow = wm * WM + l32, wrow = wn * WN + l32;
+  const int x_lane = xrow * PROW + ((hi ^ ((xrow >> 1) & 7)) << 3);  // halfs; chunk bits xor'ed per read
+  const int w_lane = wrow * PROW + ((hi ^ ((wrow >> 1) & 7)) << 3);
   half8_t fw[2][TN], fx[2][TM];
-  auto read_frags = [&](int buf, int stage, int ks) {
-    const half_t* Wb = Bs + stage * B_STAGE;
-    const half_t* Xb = As + stage * A_STAGE;
+  // par: tile of the pair (0/1), ks: k-step of the tile, stage: ring stage of the unpacked weights
+  auto read_frags = [&](int buf, const half_t* xs, const half_t* wp, int par, int stage, int ks) {
+    const int cx = (4 * par + 2 * ks) << 3;
+    if constexpr (MODE == kPlainF16) {
 #pragma unroll
-    for (int i = 0; i < TN; i++)
-      fw[buf][i] = *reinterpret_cast<const half8_t*>(Wb + lds_chunk(wn * WN + i * 32 + l32, 2 * ks + hi));
+      for (int i = 0; i < TN; i++)
+        fw[buf][i] = *reinterpret_cast<const half8_t*>(wp + (w_lane ^ cx) + i * 32 * PROW);
+    } else {
+      const half_t* Wb = Bs + stage * B_STAGE;
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+        fw[buf][i] = *reinterpret_cast<const half8_t*>(Wb + lds_chunk(wrow + i * 32, 2 * ks + hi));
+    }
 #pragma unroll
     for (int j = 0; j < TM; j++)
-      fx[buf][j] = *reinterpret_cast<const half8_t*>(Xb + lds_chunk(wm * WM + j * 32 + l32, 2 * ks + hi));
+      fx[buf][j] = *reinterpret_cast<const half8_t*>(xs + (x_lane ^ cx) + j * 32 * PROW);
   };
   auto mfma_step = [&](int buf) {
 #pragma unroll
@@ -340,72 +375,88 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[buf][i], fx[buf][j], acc[i][j], 0, 0, 0);
   };
 
-  // ---- prologue: tiles 0 and 1 into the ring, tiles 2 and 3 in flight ---------
-  issue_loads(R0);  // tile 0
-  issue_loads(R1);  // tile 1
-  issue_loads(R2);  // tile 2
-  __syncthreads();  // palettes visible
-  stage_to_lds(R0, 0);
-  issue_loads(R0);  // tile 3
+  // ---- prologue: pair 0 in slot A, weights of tiles 0 and 1 in the ring --------
+  issue_pair(XsA, WpA, 0);
+  issue_idx(WS[0]);  // tile 0
+  issue_idx(WS[1]);  // tile 1
+  __syncthreads();   // palettes visible
+  stage_to_lds(WS[0], 0);
+  issue_idx(WS[0]);  // tile 2
   if constexpr (MODE == kPalRow) {
-    const int k1 = ((rot + 1) % nk) * BK;
-    if (k1 % a.nib == 0 && nk > 1) {  // tile 1 already starts a new palette block
+    if (BK % a.nib == 0 && nk > 1) {  // tile 1 already starts a new palette block
       __syncthreads();
-      load_row_palettes(k1);
+      load_row_palettes(BK);
       __syncthreads();
     }
   }
-  stage_to_lds(R1, 1);
+  stage_to_lds(WS[1], 1);
+  issue_idx(WS[1]);  // tile 3
+  __builtin_amdgcn_s_waitcnt(kWaitVm0);
   __syncthreads();
-  read_frags(0, 0, 0);
+  read_frags(0, XsA, WpA, 0, 0, 0);
 
-  // Iteration t: MFMAs of tile t from ring stage t % 3 while tile t+2 (loaded two
-  // iterations ago) is unpacked into stage (t+2) % 3 and tile t+4 starts loading.
-  // The fragments of the next k-step are always read one step ahead, across the
-  // barrier too (stage (t+1) % 3 was completed before the previous barrier).
+  // Iteration t: MFMAs of tile t (pair t / 2) while the weights of tile t+2
+  // are unpacked into ring stage (t+2) % 3.  An even iteration starts the
+  // transfer of the next pair into the other slot (free since the barrier
+  // that ended tile t-1) and waits for it before its closing barrier, because
+  // the odd iteration reads one k-step ahead into that pair.  Index registers
+  // are refilled in odd iterations only, so the even iteration's wait covers
+  // nothing that was issued just before it.
   // The two waves of a SIMD run the two halves of an iteration in opposite
   // order (unpackers stage first, loaders run their MFMAs first), so one of
   // them is always feeding the matrix pipe while the other does VALU / LDS work.
-  auto iteration = [&](int t, RegSet& Rstage, RegSet& Rload) {
-    const int s_cur = t % NST;
-    const int s_nxt = (t + 1) % NST;
-    const int s_fill = (t + 2) % NST;
-    issue_loads(Rload);
+  int s_cur = 0, s_nxt = 1, s_fill = 2;
+  auto iteration = [&](int t, int par, half_t* xs, half_t* wp, half_t* xs_other, half_t* wp_other) {
     if constexpr (MODE == kPalRow) {
-      const int k2 = ((t + 2 + rot) % nk) * BK;
+      const int k2 = (t + 2) * BK;
       if (t + 2 < nk && k2 % a.nib == 0) {
         // lookups of tile t+1 finished before the last barrier
         load_row_palettes(k2);
         __syncthreads();
       }
     }
-    if (second) {
-      stage_to_lds(Rstage, s_fill);
-    }
+    if (par) issue_idx(WS[0]);  // tile t+3
+    auto stage_and_refill = [&]() {
+      stage_to_lds(WS[par], s_fill);
+      if (par) issue_idx(WS[1]);  // tile t+4
+    };
+    // The transfer goes out after the unpackers' LDS writes: the compiler makes
+    // every LDS write that follows a transfer wait for it to land.  The other
+    // waves write at the end of the iteration, where that wait is due anyway.
+    if (second) stage_and_refill();
+    if (par == 0) issue_pair(xs_other, wp_other, (t >> 1) + 1);
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(1, s_cur, 1);
+    read_frags(1, xs, wp, par, s_cur, 1);
     __builtin_amdgcn_sched_barrier(0);
     mfma_step(0);
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(0, s_nxt, 0);
+    if (par == 0)
+      read_frags(0, xs, wp, 1, s_nxt, 0);
+    else
+      read_frags(0, xs_other, wp_other, 0, s_nxt, 0);
     __builtin_amdgcn_sched_barrier(0);
     mfma_step(1);
     __builtin_amdgcn_sched_barrier(0);
-    if (!second) {
-      stage_to_lds(Rstage, s_fill);
-    }
+    if (!second) stage_and_refill();
+    if (par == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
     __syncthreads();
+    const int s = s_cur;
+    s_cur = s_nxt;
+    s_nxt = s_fill;
+    s_fill = s;
   };
 
-  // tile T travels in register set T % 3: iteration t stages set (t+2) % 3 and refills set (t+1) % 3
   int t = 0;
-  for (; t + 2 < nk; t += 3) {
-    iteration(t, R2, R1);
-    iteration(t + 1, R0, R2);
-    iteration(t + 2, R1, R0);
+  for (; t + 3 < nk; t += 4) {
+    iteration(t, 0, XsA, WpA, XsB, WpB);
+    iteration(t + 1, 1, XsA, WpA, XsB, WpB);
+    iteration(t + 2, 0, XsB, WpB, XsA, WpA);
+    iteration(t + 3, 1, XsB, WpB, XsA, WpA);
   }
-  if (t < nk) iteration(t, R2, R1);
-  if (t + 1 < nk) iteration(t + 1, R0, R2);
+  if (t < nk) {  // nk is even: two iterations left
+    iteration(t, 0, XsA, WpA, XsB, WpB);
+    iteration(t + 1, 1, XsA, WpA, XsB, WpB);
+  }
 
   // ---- fused epilogue: per-head RMSNorm and RoPE on the way out ---------------
   // A wave's 128 features are exactly one head, and every lane pair (l, l ^ 32)
@@ -672,7 +723,7 @@ DT_EXPORT dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K
 
   // Weights that share (qbits, nib) and meet the tiled kernel's alignment go
   // out in groups of up to kMaxWeights per launch; the rest take the generic kernel.
-  const bool x_ok = (K % BK == 0) && (ldx % 8 == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
+  const bool x_ok = (K % (2 * BK) == 0) && (ldx % 8 == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
   int i = 0;
   while (i < n_weights) {
     const dt_qx_weight& w0 = W[i];
