@@ -184,7 +184,6 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const char* wbase = reinterpret_cast<const char*>(w.data);
 
   // weight row of this thread (two threads per row; each loads and unpacks one half of the row's granule)
-  const bool b_active = (BN >= 256) || (lt < BN);
   const int b_row = lt < BN ? lt : BN - 1;
   RowCursor cur;
   int64_t pal_first_block = 0;
@@ -256,6 +255,9 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // past the end re-read the last one, harmlessly).
   auto issue_pair = [&](half_t* xs, half_t* wp, int q) {
     if (q > last_pair) q = last_pair;
+#ifdef DT_EXP_SAMEPAIR
+    q = 0;
+#endif
     const int64_t kb = (int64_t)q * (4 * BK);  // byte offset of the pair inside a row
     const char* xk = xbase + kb;
 #pragma unroll
@@ -293,42 +295,52 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     }
   };
 
-  // Unpacks the granule held in R, looks it up and writes the weights into a ring stage.
-  auto stage_to_lds = [&](const IdxSet& R, int stage) {
+  // Staging of a weight tile, in pieces that the main loop spreads between its
+  // MFMAs: unpack the 16 indices into palette byte offsets, look them up one
+  // by one, write the 16 weights as two 16-byte chunks.  Threads past the tile's
+  // last row repeat that row's work and write the same bytes again.
+  uint32_t la[16];  // palette byte offsets, then the looked-up weights
+  const char* gpal = nullptr;
+  auto unpack_indices = [&](IdxSet& R) {
+    if constexpr (MODE != kPlainF16) {
+      uint32_t idx[16];
+      unpack16_own<Q, HW>(R.b, second, idx);
+      uint32_t base = 0;
+      if constexpr (MODE == kPalGlobal)
+        gpal = wbase + R.poff;
+      else
+        base = (uint32_t)R.slot << (Q + 1);
+#pragma unroll
+      for (int j = 0; j < 16; j++) la[j] = base + (idx[j] << 1);
+    }
+  };
+  auto lookup = [&](int j) {
+    if constexpr (MODE == kPalGlobal)
+      la[j] = *reinterpret_cast<const uint16_t*>(gpal + la[j]);
+    else if constexpr (MODE != kPlainF16)
+      la[j] = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(Pal) + la[j]);
+  };
+  const int w_dst = lds_chunk(b_row, second ? 2 : 0);  // chunks c0 and c0 + 1 differ in bit 3
+  auto write_weights = [&](int stage, int h) {
     if constexpr (MODE != kPlainF16) {
       half_t* Bsd = Bs + stage * B_STAGE;
-      if (b_active) {
-        uint32_t idx[16];
-        uint32_t mine[HW];
+      const uint4_t v = {la[8 * h] | (la[8 * h + 1] << 16), la[8 * h + 2] | (la[8 * h + 3] << 16),
+                         la[8 * h + 4] | (la[8 * h + 5] << 16), la[8 * h + 6] | (la[8 * h + 7] << 16)};
+      *reinterpret_cast<uint4_t*>(&Bsd[w_dst ^ (h << 3)]) = v;
+    }
+  };
+  auto stage_to_lds = [&](IdxSet& R, int stage) {  // all at once (prologue)
+    unpack_indices(R);
 #pragma unroll
-        for (int j = 0; j < HW; j++) {
-          mine[j] = R.b[j];
-          // Pins the unpacking to this point: hoisted above the preceding barrier
-          // it would drag the wait for the index load along with it.
-          asm volatile("" : "+v"(mine[j]));
-        }
-        uint32_t g[QW];  // the granule with only this thread's dwords filled in
-        if (second) {
+    for (int j = 0; j < 16; j++) lookup(j);
+    write_weights(stage, 0);
+    write_weights(stage, 1);
+  };
+  // Makes the wait for an index load happen here rather than at its first use.
+  auto touch = [&](IdxSet& R) {
+    if constexpr (MODE != kPlainF16) {
 #pragma unroll
-          for (int j = 0; j < QW; j++) g[j] = (j >= Q / 2 && j - Q / 2 < HW) ? mine[j - Q / 2] : 0u;
-          unpack16<Q, 1>(g, idx);
-        } else {
-#pragma unroll
-          for (int j = 0; j < QW; j++) g[j] = j < HW ? mine[j] : 0u;
-          unpack16<Q, 0>(g, idx);
-        }
-        uint32_t o[8];
-        const uint16_t* pal;
-        if constexpr (MODE == kPalGlobal)
-          pal = reinterpret_cast<const uint16_t*>(wbase + R.poff);
-        else
-          pal = Pal + (R.slot << Q);
-#pragma unroll
-        for (int j = 0; j < 8; j++) o[j] = (uint32_t)pal[idx[2 * j]] | ((uint32_t)pal[idx[2 * j + 1]] << 16);
-        const int c0 = second ? 2 : 0;
-        *reinterpret_cast<uint4_t*>(&Bsd[lds_chunk(b_row, c0)]) = uint4_t{o[0], o[1], o[2], o[3]};
-        *reinterpret_cast<uint4_t*>(&Bsd[lds_chunk(b_row, c0 + 1)]) = uint4_t{o[4], o[5], o[6], o[7]};
-      }
+      for (int j = 0; j < HW; j++) asm volatile("" : "+v"(R.b[j]));
     }
   };
 
@@ -351,28 +363,17 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const int w_lane = wrow * PROW + ((hi ^ ((wrow >> 1) & 7)) << 3);
   half8_t fw[2][TN], fx[2][TM];
   // par: tile of the pair (0/1), ks: k-step of the tile, stage: ring stage of the unpacked weights
-  auto read_frags = [&](int buf, const half_t* xs, const half_t* wp, int par, int stage, int ks) {
-    const int cx = (4 * par + 2 * ks) << 3;
-    if constexpr (MODE == kPlainF16) {
-#pragma unroll
-      for (int i = 0; i < TN; i++)
-        fw[buf][i] = *reinterpret_cast<const half8_t*>(wp + (w_lane ^ cx) + i * 32 * PROW);
-    } else {
-      const half_t* Wb = Bs + stage * B_STAGE;
-#pragma unroll
-      for (int i = 0; i < TN; i++)
-        fw[buf][i] = *reinterpret_cast<const half8_t*>(Wb + lds_chunk(wrow + i * 32, 2 * ks + hi));
-    }
-#pragma unroll
-    for (int j = 0; j < TM; j++)
-      fx[buf][j] = *reinterpret_cast<const half8_t*>(xs + (x_lane ^ cx) + j * 32 * PROW);
+  auto read_w = [&](int buf, int i, const half_t* wp, int par, int stage, int ks) {
+    if constexpr (MODE == kPlainF16)
+      fw[buf][i] = *reinterpret_cast<const half8_t*>(wp + (w_lane ^ ((4 * par + 2 * ks) << 3)) + i * 32 * PROW);
+    else
+      fw[buf][i] = *reinterpret_cast<const half8_t*>(Bs + stage * B_STAGE + lds_chunk(wrow + i * 32, 2 * ks + hi));
   };
-  auto mfma_step = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < TN; i++)
-#pragma unroll
-      for (int j = 0; j < TM; j++)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[buf][i], fx[buf][j], acc[i][j], 0, 0, 0);
+  auto read_x = [&](int buf, int j, const half_t* xs, int par, int ks) {
+    fx[buf][j] = *reinterpret_cast<const half8_t*>(xs + (x_lane ^ ((4 * par + 2 * ks) << 3)) + j * 32 * PROW);
+  };
+  auto mfma = [&](int buf, int i, int j) {
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[buf][i], fx[buf][j], acc[i][j], 0, 0, 0);
   };
 
   // ---- prologue: pair 0 in slot A, weights of tiles 0 and 1 in the ring --------
@@ -393,7 +394,10 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   issue_idx(WS[1]);  // tile 3
   __builtin_amdgcn_s_waitcnt(kWaitVm0);
   __syncthreads();
-  read_frags(0, XsA, WpA, 0, 0, 0);
+#pragma unroll
+  for (int i = 0; i < TN; i++) read_w(0, i, WpA, 0, 0, 0);
+#pragma unroll
+  for (int j = 0; j < TM; j++) read_x(0, j, XsA, 0, 0);
 
   // Iteration t: MFMAs of tile t (pair t / 2) while the weights of tile t+2
   // are unpacked into ring stage (t+2) % 3.  An even iteration starts the
@@ -402,9 +406,12 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // the odd iteration reads one k-step ahead into that pair.  Index registers
   // are refilled in odd iterations only, so the even iteration's wait covers
   // nothing that was issued just before it.
-  // The two waves of a SIMD run the two halves of an iteration in opposite
-  // order (unpackers stage first, loaders run their MFMAs first), so one of
-  // them is always feeding the matrix pipe while the other does VALU / LDS work.
+  //
+  // A wave issues in order, and an LDS instruction occupies it for tens of
+  // clocks, so the iteration is written as 16 slots of one MFMA followed by
+  // a share of the LDS and VALU work: the fragment reads of the next k-step,
+  // the palette lookups and the weight writes all issue while an MFMA of the
+  // same wave (or of the wave it shares the SIMD with) is executing.
   int s_cur = 0, s_nxt = 1, s_fill = 2;
   auto iteration = [&](int t, int par, half_t* xs, half_t* wp, half_t* xs_other, half_t* wp_other) {
     if constexpr (MODE == kPalRow) {
@@ -415,30 +422,55 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         __syncthreads();
       }
     }
-    if (par) issue_idx(WS[0]);  // tile t+3
-    auto stage_and_refill = [&]() {
-      stage_to_lds(WS[par], s_fill);
-      if (par) issue_idx(WS[1]);  // tile t+4
-    };
-    // The transfer goes out after the unpackers' LDS writes: the compiler makes
-    // every LDS write that follows a transfer wait for it to land.  The other
-    // waves write at the end of the iteration, where that wait is due anyway.
-    if (second) stage_and_refill();
-    if (par == 0) issue_pair(xs_other, wp_other, (t >> 1) + 1);
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(1, xs, wp, par, s_cur, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma_step(0);
-    __builtin_amdgcn_sched_barrier(0);
+    IdxSet& R = WS[par];
+    // the wait for the indices comes before the transfer goes out: a wait with
+    // the transfer outstanding would last until it lands
+    touch(R);
     if (par == 0)
-      read_frags(0, xs, wp, 1, s_nxt, 0);
+      issue_pair(xs_other, wp_other, (t >> 1) + 1);
     else
-      read_frags(0, xs_other, wp_other, 0, s_nxt, 0);
+      issue_idx(WS[0]);  // tile t+3
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step(1);
+    unpack_indices(R);
+    if (par) issue_idx(WS[1]);  // tile t+4
+    // fragments of tile t+1, k-step 0
+    const half_t* xs_n = par == 0 ? xs : xs_other;
+    const half_t* wp_n = par == 0 ? wp : wp_other;
+    constexpr int NM = TN * TM;  // MFMAs per k-step = slots per phase
+    // k-step 0: the fragments of k-step 1 first, then the first 8 lookups
+    constexpr int N0 = TN + TM + 8;
+    auto op0 = [&](int k) {
+      if (k < TN) read_w(1, k, wp, par, s_cur, 1);
+      else if (k < TN + TM) read_x(1, k - TN, xs, par, 1);
+      else lookup(k - TN - TM);
+    };
+    // k-step 1: the other 8 lookups, the next tile's first fragments (every
+    // k-step 0 MFMA has been issued, so their registers are free), the writes
+    constexpr int N1 = 8 + TN + TM + 2;
+    auto op1 = [&](int k) {
+      if (k < 8) lookup(8 + k);
+      else if (k < 8 + TN) read_w(0, k - 8, wp_n, par ^ 1, s_nxt, 0);
+      else if (k < 8 + TN + TM) read_x(0, k - 8 - TN, xs_n, par ^ 1, 0);
+      else write_weights(s_fill, k - 8 - TN - TM);
+    };
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+      __builtin_amdgcn_sched_barrier(0);
+      mfma(0, m / TM, m % TM);
+#pragma unroll
+      for (int k = m * N0 / NM; k < (m + 1) * N0 / NM; k++) op0(k);
+    }
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+      __builtin_amdgcn_sched_barrier(0);
+      mfma(1, m / TM, m % TM);
+#pragma unroll
+      for (int k = m * N1 / NM; k < (m + 1) * N1 / NM; k++) op1(k);
+    }
     __builtin_amdgcn_sched_barrier(0);
-    if (!second) stage_and_refill();
+#ifndef DT_EXP_NOWAIT
     if (par == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
+#endif
     __syncthreads();
     const int s = s_cur;
     s_cur = s_nxt;
