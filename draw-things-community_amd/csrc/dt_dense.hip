@@ -10,6 +10,8 @@
 // LDS is double-buffered; the global loads of tile t+1 are issued before the
 // MFMAs of tile t and its unpack/lookup runs after them, so one barrier per
 // K-tile and the unpack VALU/LDS work overlaps the matrix pipe.
+#include <numeric>
+
 #include "dt_common.h"
 #include "dt_layout.h"
 #include "dt_qkprep.h"
@@ -23,7 +25,7 @@ constexpr int kPalLdsBytes = 32768;
 
 enum PalMode : int {
   kPalShared = 0,  // palettes of every block the tile's rows touch, loaded once, slot = block - first block
-  kPalRow = 1,     // nib < K, K % nib == 0: one palette per row, reloaded every nib columns
+  kPalRow = 1,     // one palette per row in a transposed table, a row's column rewritten where its block changes
   kPalGlobal = 2,  // lookups go to global memory (any layout)
   kPlainF16 = 3    // weight is plain fp16, no palette
 };
@@ -47,6 +49,7 @@ struct DenseArgs {
   int64_t ldx;
   int32_t m, k;
   int32_t nib;
+  int32_t pal_step;  // K-tiles between columns at which a row can enter a new palette block: gcd(K, nib) / 32
   int32_t n_weights;
   int32_t tiles_m, tiles_n;
   DenseWeight w[kMaxWeights];
@@ -226,20 +229,33 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       reinterpret_cast<uint32_t*>(Pal)[i] = src[e];
     }
   }
-  auto load_row_palettes = [&](int k0) {
-    // kPalRow: block of row n at column k0 is n * (K / nib) + k0 / nib
-    const int per_pal = 1 << (Q - 1);
-    const int bpr = K / a.nib;
-    for (int i = tid; i < BN * per_pal; i += 512) {
-      int row = i / per_pal, e = i - row * per_pal;
-      int gn = n0 + row;
-      if (gn >= w.n) gn = w.n - 1;
-      int64_t blk = (int64_t)gn * bpr + k0 / a.nib;
-      const uint32_t* src = reinterpret_cast<const uint32_t*>(w.data + palette_offset(lay, blk));
-      reinterpret_cast<uint32_t*>(Pal)[i] = src[e];
+  // kPalRow: Pal is a table [64-row group][entry][row % 64] of fp16, so the 64
+  // lanes of a wave (64 consecutive rows, one entry each) read 64 consecutive
+  // halfs of some entry rows: two lanes share a bank, nothing worse.  Each of a
+  // row's two threads keeps half of the row's column current.
+  const int pal_col = (b_row >> 6) * (128 << Q) + (b_row & 63) * 2;  // byte offset of this row's column
+  auto fill_pal_column = [&](int64_t blk) {
+    constexpr int ND = (1 << Q) / 4;  // dwords of palette per thread
+    const uint32_t* src =
+        reinterpret_cast<const uint32_t*>(w.data + palette_offset(lay, blk)) + (second ? ND : 0);
+    char* dst = reinterpret_cast<char*>(Pal) + pal_col + (second ? (64 << Q) : 0);
+#pragma unroll
+    for (int d = 0; d < ND; d++) {
+      const uint32_t v = src[d];
+      *reinterpret_cast<uint16_t*>(dst + (2 * d) * 128) = (uint16_t)v;
+      *reinterpret_cast<uint16_t*>(dst + (2 * d + 1) * 128) = (uint16_t)(v >> 16);
     }
   };
-  if constexpr (MODE == kPalRow) load_row_palettes(0);
+  int gn_row = n0 + b_row;  // this thread's weight row
+  if (gn_row >= w.n) gn_row = w.n - 1;
+  // rewrites the column if the row enters a new block at K-tile `tile`
+  auto refresh_pal_column = [&](int tile) {
+    const int64_t e = (int64_t)gn_row * K + (int64_t)tile * BK;
+    const int64_t blk = e / a.nib;
+    if (e == blk * a.nib) fill_pal_column(blk);
+  };
+  int next_pal_tile = a.pal_step;  // next K-tile at which some row may change block
+  if constexpr (MODE == kPalRow) fill_pal_column(((int64_t)gn_row * K) / a.nib);
 
   // ---- staging --------------------------------------------------------------
   struct IdxSet {
@@ -305,13 +321,18 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     if constexpr (MODE != kPlainF16) {
       uint32_t idx[16];
       unpack16_own<Q, HW>(R.b, second, idx);
-      uint32_t base = 0;
-      if constexpr (MODE == kPalGlobal)
-        gpal = wbase + R.poff;
-      else
-        base = (uint32_t)R.slot << (Q + 1);
+      if constexpr (MODE == kPalRow) {
 #pragma unroll
-      for (int j = 0; j < 16; j++) la[j] = base + (idx[j] << 1);
+        for (int j = 0; j < 16; j++) la[j] = (uint32_t)pal_col + (idx[j] << 7);
+      } else {
+        uint32_t base = 0;
+        if constexpr (MODE == kPalGlobal)
+          gpal = wbase + R.poff;
+        else
+          base = (uint32_t)R.slot << (Q + 1);
+#pragma unroll
+        for (int j = 0; j < 16; j++) la[j] = base + (idx[j] << 1);
+      }
     }
   };
   auto lookup = [&](int j) {
@@ -384,9 +405,10 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   stage_to_lds(WS[0], 0);
   issue_idx(WS[0]);  // tile 2
   if constexpr (MODE == kPalRow) {
-    if (BK % a.nib == 0 && nk > 1) {  // tile 1 already starts a new palette block
+    if (next_pal_tile == 1) {  // tile 1 may already start a new palette block
       __syncthreads();
-      load_row_palettes(BK);
+      refresh_pal_column(1);
+      next_pal_tile += a.pal_step;
       __syncthreads();
     }
   }
@@ -415,10 +437,10 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   int s_cur = 0, s_nxt = 1, s_fill = 2;
   auto iteration = [&](int t, int par, half_t* xs, half_t* wp, half_t* xs_other, half_t* wp_other) {
     if constexpr (MODE == kPalRow) {
-      const int k2 = (t + 2) * BK;
-      if (t + 2 < nk && k2 % a.nib == 0) {
+      if (t + 2 == next_pal_tile) {
         // lookups of tile t+1 finished before the last barrier
-        load_row_palettes(k2);
+        if (t + 2 < nk) refresh_pal_column(t + 2);
+        next_pal_tile += a.pal_step;
         __syncthreads();
       }
     }
@@ -438,20 +460,24 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     const half_t* wp_n = par == 0 ? wp : wp_other;
     constexpr int NM = TN * TM;  // MFMAs per k-step = slots per phase
     // k-step 0: the fragments of k-step 1 first, then the first 8 lookups
-    constexpr int N0 = TN + TM + 8;
+    constexpr int NL = MODE == kPlainF16 ? 0 : 8;  // lookups per phase
+    constexpr int NF = TN + TM;                    // fragment reads per phase
+    constexpr int N0 = NF + NL;
     auto op0 = [&](int k) {
       if (k < TN) read_w(1, k, wp, par, s_cur, 1);
-      else if (k < TN + TM) read_x(1, k - TN, xs, par, 1);
-      else lookup(k - TN - TM);
+      else if (k < NF) read_x(1, k - TN, xs, par, 1);
+      else lookup(k - NF);
     };
-    // k-step 1: the other 8 lookups, the next tile's first fragments (every
-    // k-step 0 MFMA has been issued, so their registers are free), the writes
-    constexpr int N1 = 8 + TN + TM + 2;
+    // k-step 1: half of the remaining lookups, the next tile's first fragments
+    // (every k-step 0 MFMA has been issued, so their registers are free), the
+    // other lookups, the writes
+    constexpr int N1 = NL + NF + (NL ? 2 : 0);
     auto op1 = [&](int k) {
-      if (k < 8) lookup(8 + k);
-      else if (k < 8 + TN) read_w(0, k - 8, wp_n, par ^ 1, s_nxt, 0);
-      else if (k < 8 + TN + TM) read_x(0, k - 8 - TN, xs_n, par ^ 1, 0);
-      else write_weights(s_fill, k - 8 - TN - TM);
+      if (k < NL / 2) lookup(8 + k);
+      else if (k < NL / 2 + TN) read_w(0, k - NL / 2, wp_n, par ^ 1, s_nxt, 0);
+      else if (k < NL / 2 + NF) read_x(0, k - NL / 2 - TN, xs_n, par ^ 1, 0);
+      else if (k < NL + NF) lookup(8 + k - NF);
+      else write_weights(s_fill, k - NL - NF);
     };
 #pragma unroll
     for (int m = 0; m < NM; m++) {
@@ -470,6 +496,9 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     __builtin_amdgcn_sched_barrier(0);
 #ifndef DT_EXP_NOWAIT
     if (par == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
+#endif
+#ifdef DT_EXP_NOBAR
+    if (par == 1)
 #endif
     __syncthreads();
     const int s = s_cur;
@@ -709,9 +738,9 @@ static dt_status launch_tiled_q(hipStream_t s, const DenseArgs& a, int qbits, in
 static int choose_pal_mode(int qbits, int nib, int64_t K, int BN) {
   if (qbits == 16) return kPlainF16;
   const int64_t pal_bytes = (int64_t)2 << qbits;
+  if ((int64_t)BN * pal_bytes <= kPalLdsBytes) return kPalRow;
   const int64_t shared_count = ((int64_t)BN * K) / nib + 2;
   if (shared_count * pal_bytes <= kPalLdsBytes) return kPalShared;
-  if (nib < K && K % nib == 0 && (int64_t)BN * pal_bytes <= kPalLdsBytes) return kPalRow;
   return kPalGlobal;
 }
 
@@ -820,6 +849,7 @@ DT_EXPORT dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K
     a.m = (int32_t)M;
     a.k = (int32_t)K;
     a.nib = w0.qbits == 16 ? 32 : w0.nib;
+    a.pal_step = (int32_t)(std::gcd((int64_t)K, (int64_t)a.nib) / BK);
     a.tiles_m = (int)((M + BM - 1) / BM);
     int tiles_n = 0, cnt = 0;
     const int first = i;
