@@ -82,7 +82,12 @@ __device__ __forceinline__ int lds_chunk(int row, int c) { return row * BK + ((c
 // consecutive rows of one chunk column on 16 distinct 16-byte bank groups.
 __device__ __forceinline__ int pair_chunk(int row, int slot) { return slot ^ ((row >> 1) & 7); }
 
-constexpr int kWaitVm0 = 0x0f70;  // s_waitcnt vmcnt(0), other counters untouched
+constexpr int kWaitVm0Lgkm0 = 0x0070;  // s_waitcnt vmcnt(0) lgkmcnt(0)
+constexpr int kWaitLgkm0 = 0xc07f;     // s_waitcnt lgkmcnt(0)
+
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
 
 // One wave-wide memory -> LDS transfer: lane l's 16 bytes at g land at LDS
 // address lds + 16 * l (lds wave-uniform).
@@ -125,7 +130,8 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   __shared__ __attribute__((aligned(1024))) half_t WpA[MODE == kPlainF16 ? BN * PROW : 8];
   __shared__ __attribute__((aligned(1024))) half_t WpB[MODE == kPlainF16 ? BN * PROW : 8];
   __shared__ __attribute__((aligned(16))) half_t Bs[MODE == kPlainF16 ? 8 : NST * B_STAGE];
-  __shared__ __attribute__((aligned(16))) uint16_t Pal[(MODE == kPalShared || MODE == kPalRow) ? kPalLdsBytes / 2 : 8];
+  // the strictest alignment puts the palettes first in LDS, where their address fits an instruction offset
+  __shared__ __attribute__((aligned(4096))) uint16_t Pal[(MODE == kPalShared || MODE == kPalRow) ? kPalLdsBytes / 2 : 8];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -267,24 +273,23 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const int last_pair = nk / 2 - 1;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
 
-  // Starts the memory -> LDS transfer of K-tile pair q into a pair slot (pairs
-  // past the end re-read the last one, harmlessly).
-  auto issue_pair = [&](half_t* xs, half_t* wp, int q) {
+  // Part i (of AP + BP) of the memory -> LDS transfer of K-tile pair q into a
+  // pair slot (pairs past the end re-read the last one, harmlessly).
+  auto issue_pair_part = [&](half_t* xs, half_t* wp, int q, int i) {
     if (q > last_pair) q = last_pair;
-#ifdef DT_EXP_SAMEPAIR
-    q = 0;
+#ifdef DT_EXP_NODMA
+    if (q > 0) return;
 #endif
     const int64_t kb = (int64_t)q * (4 * BK);  // byte offset of the pair inside a row
-    const char* xk = xbase + kb;
-#pragma unroll
-    for (int i = 0; i < AP; i++)
-      load_to_lds_16(xk + a_off[i], xs + (wave_u * AP + i) * 512);
-    if constexpr (MODE == kPlainF16) {
-      const char* wk = wbase + kb;
-#pragma unroll
-      for (int i = 0; i < BP; i++)
-        load_to_lds_16(wk + bf_off[i], wp + (wave_u * BP + i) * 512);
+    if (i < AP) {
+      load_to_lds_16(xbase + kb + a_off[i], xs + (wave_u * AP + i) * 512);
+    } else if constexpr (MODE == kPlainF16) {
+      load_to_lds_16(wbase + kb + bf_off[i - AP], wp + (wave_u * BP + i - AP) * 512);
     }
+  };
+  auto issue_pair = [&](half_t* xs, half_t* wp, int q) {
+#pragma unroll
+    for (int i = 0; i < AP + BP; i++) issue_pair_part(xs, wp, q, i);
   };
 
   // Loads the indices of the tile the cursor points at (the last tile is re-read
@@ -316,23 +321,21 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // by one, write the 16 weights as two 16-byte chunks.  Threads past the tile's
   // last row repeat that row's work and write the same bytes again.
   uint32_t la[16];  // palette byte offsets, then the looked-up weights
+  uint32_t be[HW + 1];
   const char* gpal = nullptr;
-  auto unpack_indices = [&](IdxSet& R) {
+  uint32_t pal_base = 0;
+  // piece 0 also turns the index dwords into a bit string; piece p yields offsets 4p .. 4p+3
+  auto unpack_piece = [&](IdxSet& R, int p) {
     if constexpr (MODE != kPlainF16) {
-      uint32_t idx[16];
-      unpack16_own<Q, HW>(R.b, second, idx);
-      if constexpr (MODE == kPalRow) {
-#pragma unroll
-        for (int j = 0; j < 16; j++) la[j] = (uint32_t)pal_col + (idx[j] << 7);
-      } else {
-        uint32_t base = 0;
-        if constexpr (MODE == kPalGlobal)
-          gpal = wbase + R.poff;
-        else
-          base = (uint32_t)R.slot << (Q + 1);
-#pragma unroll
-        for (int j = 0; j < 16; j++) la[j] = base + (idx[j] << 1);
+      if (p == 0) {
+        own_bits<Q, HW>(R.b, second, be);
+        if constexpr (MODE == kPalRow) pal_base = (uint32_t)pal_col;
+        else if constexpr (MODE == kPalGlobal) gpal = wbase + R.poff;
+        else pal_base = (uint32_t)R.slot << (Q + 1);
       }
+#pragma unroll
+      for (int j = 4 * p; j < 4 * p + 4; j++)
+        la[j] = pal_base | (own_index<Q, HW>(be, j) << (MODE == kPalRow ? 7 : 1));  // disjoint bits
     }
   };
   auto lookup = [&](int j) {
@@ -341,17 +344,22 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     else if constexpr (MODE != kPlainF16)
       la[j] = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(Pal) + la[j]);
   };
-  const int w_dst = lds_chunk(b_row, second ? 2 : 0);  // chunks c0 and c0 + 1 differ in bit 3
+  // Written as assembly: the compiler makes every LDS store it knows of wait
+  // for all memory -> LDS transfers in flight, which would stall the even
+  // iterations until the next pair has landed.  The closing s_waitcnt of an
+  // iteration covers these stores.
+  const uint32_t w_dst = lds_address(Bs) + 2u * (uint32_t)lds_chunk(b_row, second ? 2 : 0);
   auto write_weights = [&](int stage, int h) {
     if constexpr (MODE != kPlainF16) {
-      half_t* Bsd = Bs + stage * B_STAGE;
       const uint4_t v = {la[8 * h] | (la[8 * h + 1] << 16), la[8 * h + 2] | (la[8 * h + 3] << 16),
                          la[8 * h + 4] | (la[8 * h + 5] << 16), la[8 * h + 6] | (la[8 * h + 7] << 16)};
-      *reinterpret_cast<uint4_t*>(&Bsd[w_dst ^ (h << 3)]) = v;
+      const uint32_t addr = (w_dst + (uint32_t)(stage * B_STAGE * 2)) ^ (uint32_t)(h << 4);  // chunks c0, c0 + 1 differ in bit 4
+      asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
     }
   };
   auto stage_to_lds = [&](IdxSet& R, int stage) {  // all at once (prologue)
-    unpack_indices(R);
+#pragma unroll
+    for (int p = 0; p < 4; p++) unpack_piece(R, p);
 #pragma unroll
     for (int j = 0; j < 16; j++) lookup(j);
     write_weights(stage, 0);
@@ -385,12 +393,18 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   half8_t fw[2][TN], fx[2][TM];
   // par: tile of the pair (0/1), ks: k-step of the tile, stage: ring stage of the unpacked weights
   auto read_w = [&](int buf, int i, const half_t* wp, int par, int stage, int ks) {
+#ifdef DT_EXP_NOREAD
+    if (buf >= 0) return;
+#endif
     if constexpr (MODE == kPlainF16)
       fw[buf][i] = *reinterpret_cast<const half8_t*>(wp + (w_lane ^ ((4 * par + 2 * ks) << 3)) + i * 32 * PROW);
     else
       fw[buf][i] = *reinterpret_cast<const half8_t*>(Bs + stage * B_STAGE + lds_chunk(wrow + i * 32, 2 * ks + hi));
   };
   auto read_x = [&](int buf, int j, const half_t* xs, int par, int ks) {
+#ifdef DT_EXP_NOREAD
+    if (buf >= 0) return;
+#endif
     fx[buf][j] = *reinterpret_cast<const half8_t*>(xs + (x_lane ^ ((4 * par + 2 * ks) << 3)) + j * 32 * PROW);
   };
   auto mfma = [&](int buf, int i, int j) {
@@ -414,7 +428,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   }
   stage_to_lds(WS[1], 1);
   issue_idx(WS[1]);  // tile 3
-  __builtin_amdgcn_s_waitcnt(kWaitVm0);
+  __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < TN; i++) read_w(0, i, WpA, 0, 0, 0);
@@ -445,57 +459,80 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       }
     }
     IdxSet& R = WS[par];
-    // the wait for the indices comes before the transfer goes out: a wait with
-    // the transfer outstanding would last until it lands
+    // the wait for the indices comes here, before the transfer goes out: a
+    // wait with the transfer outstanding would last until it lands
     touch(R);
-    if (par == 0)
-      issue_pair(xs_other, wp_other, (t >> 1) + 1);
-    else
-      issue_idx(WS[0]);  // tile t+3
-    __builtin_amdgcn_sched_barrier(0);
-    unpack_indices(R);
-    if (par) issue_idx(WS[1]);  // tile t+4
-    // fragments of tile t+1, k-step 0
-    const half_t* xs_n = par == 0 ? xs : xs_other;
+    if (par) issue_idx(WS[0]);  // tile t+3
+    const half_t* xs_n = par == 0 ? xs : xs_other;  // fragments of tile t+1, k-step 0
     const half_t* wp_n = par == 0 ? wp : wp_other;
     constexpr int NM = TN * TM;  // MFMAs per k-step = slots per phase
-    // k-step 0: the fragments of k-step 1 first, then the first 8 lookups
-    constexpr int NL = MODE == kPlainF16 ? 0 : 8;  // lookups per phase
-    constexpr int NF = TN + TM;                    // fragment reads per phase
-    constexpr int N0 = NF + NL;
-    auto op0 = [&](int k) {
-      if (k < TN) read_w(1, k, wp, par, s_cur, 1);
-      else if (k < NF) read_x(1, k - TN, xs, par, 1);
-      else lookup(k - NF);
+    constexpr int NF = TN + TM;  // fragment reads per phase
+    constexpr bool packed = MODE != kPlainF16;
+    // Phase 0 (k-step 0): the fragments of k-step 1, one every third place;
+    // between them the parts of the transfer (even iterations), the unpacking,
+    // the refill of the index registers (odd iterations), the first 8 lookups.
+    const int nd = par == 0 ? AP + BP : 0;
+    const int ns0 = nd + (packed ? 4 + par + 8 : 0);
+    auto stage0 = [&](int s) {
+      if (s < nd) { issue_pair_part(xs_other, wp_other, (t >> 1) + 1, s); return; }
+      s -= nd;
+      if (!packed) return;
+      if (s < 4) { unpack_piece(R, s); return; }
+      s -= 4;
+      if (par) {
+        if (s == 0) { issue_idx(WS[1]); return; }  // tile t+4
+        s -= 1;
+      }
+      if (s < 8) lookup(s);
     };
-    // k-step 1: half of the remaining lookups, the next tile's first fragments
-    // (every k-step 0 MFMA has been issued, so their registers are free), the
-    // other lookups, the writes
-    constexpr int N1 = NL + NF + (NL ? 2 : 0);
-    auto op1 = [&](int k) {
-      if (k < NL / 2) lookup(8 + k);
-      else if (k < NL / 2 + TN) read_w(0, k - NL / 2, wp_n, par ^ 1, s_nxt, 0);
-      else if (k < NL / 2 + NF) read_x(0, k - NL / 2 - TN, xs_n, par ^ 1, 0);
-      else if (k < NL + NF) lookup(8 + k - NF);
-      else write_weights(s_fill, k - NL - NF);
+    // Phase 1 (k-step 1): the next tile's first fragments (every k-step 0
+    // MFMA has been issued, so their registers are free), the other lookups,
+    // the two weight writes.
+    const int ns1 = packed ? 10 : 0;
+    auto stage1 = [&](int s) {
+      if (!packed) return;
+      if (s < 8) lookup(8 + s);
+      else if (s < 10) write_weights(s_fill, s - 8);
     };
+    auto read0 = [&](int r) {
+      if (r < TN) read_w(1, r, wp, par, s_cur, 1);
+      else read_x(1, r - TN, xs, par, 1);
+    };
+    auto read1 = [&](int r) {
+      if (r < TN) read_w(0, r, wp_n, par ^ 1, s_nxt, 0);
+      else read_x(0, r - TN, xs_n, par ^ 1, 0);
+    };
+    // place k of a phase: a read at every third place while reads last, stage parts elsewhere
+    auto place = [&](int k, int ns, auto&& rd, auto&& st) {
+      if (k < 3 * NF) {
+        if (k % 3 == 0) rd(k / 3);
+        else if ((k / 3) * 2 + k % 3 - 1 < ns) st((k / 3) * 2 + k % 3 - 1);
+      } else if (k - NF < ns) {
+        st(k - NF);
+      }
+    };
+    const int n0 = NF + (ns0 > 2 * NF ? ns0 : 2 * NF);
+    const int n1 = NF + (ns1 > 2 * NF ? ns1 : 2 * NF);
 #pragma unroll
     for (int m = 0; m < NM; m++) {
       __builtin_amdgcn_sched_barrier(0);
       mfma(0, m / TM, m % TM);
 #pragma unroll
-      for (int k = m * N0 / NM; k < (m + 1) * N0 / NM; k++) op0(k);
+      for (int k = m * n0 / NM; k < (m + 1) * n0 / NM; k++) place(k, ns0, read0, stage0);
     }
 #pragma unroll
     for (int m = 0; m < NM; m++) {
       __builtin_amdgcn_sched_barrier(0);
       mfma(1, m / TM, m % TM);
 #pragma unroll
-      for (int k = m * N1 / NM; k < (m + 1) * N1 / NM; k++) op1(k);
+      for (int k = m * n1 / NM; k < (m + 1) * n1 / NM; k++) place(k, ns1, read1, stage1);
     }
     __builtin_amdgcn_sched_barrier(0);
 #ifndef DT_EXP_NOWAIT
-    if (par == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
+    if (par == 0)
+      __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+    else
+      __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
 #endif
 #ifdef DT_EXP_NOBAR
     if (par == 1)

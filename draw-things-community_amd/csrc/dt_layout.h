@@ -112,10 +112,12 @@ __device__ __forceinline__ void unpack16(const uint32_t (&raw)[Q], uint32_t (&id
 // The same 16 indices from the HW = (Q + 1) / 2 dwords that hold them: `own`
 // starts at dword Q / 2 * upper of the granule, where the upper half begins at
 // bit 0 (even Q) or bit 16 (odd Q).  `upper` is a run-time value, so threads
-// working on either half share one instruction stream.
+// working on either half share one instruction stream.  Two steps, so that a
+// caller can spread the extractions out: own_bits() turns the dwords into one
+// big-endian bit string starting at the half's first index, own_index() cuts
+// index j out of it.
 template <int Q, int HW>
-__device__ __forceinline__ void unpack16_own(const uint32_t (&own)[HW], bool upper, uint32_t (&idx)[16]) {
-  uint32_t be[HW + 1];
+__device__ __forceinline__ void own_bits(const uint32_t (&own)[HW], bool upper, uint32_t (&be)[HW + 1]) {
 #pragma unroll
   for (int i = 0; i < HW; i++) be[i] = __builtin_bswap32(own[i]);
   be[HW] = 0;
@@ -123,17 +125,14 @@ __device__ __forceinline__ void unpack16_own(const uint32_t (&own)[HW], bool upp
 #pragma unroll
     for (int i = 0; i < HW; i++) be[i] = upper ? __builtin_amdgcn_alignbit(be[i], be[i + 1], 16) : be[i];
   }
-#pragma unroll
-  for (int j = 0; j < 16; j++) {
-    const int bit = j * Q;
-    const int word = bit >> 5;
-    const int off = bit & 31;
-    if (off + Q <= 32) {
-      idx[j] = (be[word] >> (32 - off - Q)) & ((1u << Q) - 1);
-    } else {
-      idx[j] = __builtin_amdgcn_alignbit(be[word], be[word + 1], 64 - off - Q) & ((1u << Q) - 1);
-    }
-  }
+}
+template <int Q, int HW>
+__device__ __forceinline__ uint32_t own_index(const uint32_t (&be)[HW + 1], int j) {
+  const int bit = j * Q;
+  const int word = bit >> 5;
+  const int off = bit & 31;
+  if (off + Q <= 32) return (be[word] >> (32 - off - Q)) & ((1u << Q) - 1);
+  return __builtin_amdgcn_alignbit(be[word], be[word + 1], 64 - off - Q) & ((1u << Q) - 1);
 }
 #endif
 
