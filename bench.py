@@ -100,6 +100,14 @@ def main():
         pkg.dense_multi(img, [w["x_q"], w["x_k"], w["x_v"]], [bias["x_q"], bias["x_k"], bias["x_v"]], outs=views(T, S),
                         epilogues=epi_x)
 
+    # the context and image projections are independent Dense ops: enqueued together they share one launch
+    def k_qkv():
+        pkg.dense_grouped([
+            dict(x=img, weights=[w["x_q"], w["x_k"], w["x_v"]], biases=[bias["x_q"], bias["x_k"], bias["x_v"]],
+                 outs=views(T, S), epilogues=epi_x),
+            dict(x=ctx, weights=[w["c_q"], w["c_k"], w["c_v"]], biases=[bias["c_q"], bias["c_k"], bias["c_v"]],
+                 outs=views(0, T), epilogues=epi_c)])
+
     def k_prep():
         for t4, gc, gx in ((q4, gamma["c_q"], gamma["x_q"]), (k4, gamma["c_k"], gamma["x_k"])):
             pkg.qk_norm_rope_(t4[:, :T], gc, 1e-6, True, rot=rot, rot_pos0=0)
@@ -109,12 +117,11 @@ def main():
         pkg.sdpa_segments([q4], [k4], [v4], scale, out=att)
 
     def k_out():
-        pkg.dense_multi(att2[:T], [w["c_o"]], [bias["c_o"]], outs=[out_c])
-        pkg.dense_multi(att2[T:], [w["x_o"]], [bias["x_o"]], outs=[out_x])
+        pkg.dense_grouped([dict(x=att2[T:], weights=[w["x_o"]], biases=[bias["x_o"]], outs=[out_x]),
+                           dict(x=att2[:T], weights=[w["c_o"]], biases=[bias["c_o"]], outs=[out_c])])
 
     def step():
-        k_qkv_text()
-        k_qkv_image()
+        k_qkv()
         k_sdpa()
         k_out()
 
@@ -152,7 +159,9 @@ def main():
         return e0.elapsed_time(e1) / iters
 
     it = args.kernel_iters
+    time_kernel(k_sdpa, 2)  # first use of timing events: not measured
     ms = {
+        "dense_qkv_grouped": time_kernel(k_qkv, it),
         "dense_qkv_image_M4096": time_kernel(k_qkv_image, it),
         "dense_qkv_text_M512": time_kernel(k_qkv_text, it),
         "qk_norm_rope": time_kernel(k_prep, it),  # the standalone pass; not part of the step (fused into the QKV epilogue)
@@ -179,7 +188,8 @@ def main():
         "dense_plainf16_M4608_N3072": {"ms": ms["dense_plainf16_M4608_N3072"], "tflops": tf(2.0 * S * C * C, ms["dense_plainf16_M4608_N3072"])},
         "dense_qkv_image_M4096": {"ms": ms["dense_qkv_image_M4096"], "tflops": tf(2.0 * HW * C * 3 * C, ms["dense_qkv_image_M4096"])},
         "dense_qkv_text_M512": {"ms": ms["dense_qkv_text_M512"], "tflops": tf(2.0 * T * C * 3 * C, ms["dense_qkv_text_M512"])},
-        "dense_out_2x": {"ms": ms["dense_out_2x"], "tflops": tf(2.0 * S * C * C, ms["dense_out_2x"])},
+        "dense_qkv_text+image_one_launch": {"ms": ms["dense_qkv_grouped"], "tflops": tf(2.0 * S * C * 3 * C, ms["dense_qkv_grouped"])},
+        "dense_out_text+image_one_launch": {"ms": ms["dense_out_2x"], "tflops": tf(2.0 * S * C * C, ms["dense_out_2x"])},
         "qk_norm_rope": {"ms": ms["qk_norm_rope"], "gbs": 2 * 2 * S * C * 2 / (ms["qk_norm_rope"] * 1e-3) / 1e9},
     }
     for k in kernels.values():
@@ -188,12 +198,12 @@ def main():
         k["ms"] = round(k["ms"], 4)
 
     # dominant kernel of the step (by time): roofline against the fp16 MFMA peak
-    dense_ms = ms["dense_qkv_image_M4096"] + ms["dense_qkv_text_M512"] + ms["dense_out_2x"]
-    if ms["sdpa_S4608"] >= ms["dense_qkv_image_M4096"]:
+    dense_ms = ms["dense_qkv_grouped"] + ms["dense_out_2x"]
+    if ms["sdpa_S4608"] >= ms["dense_qkv_grouped"]:
         dom, dom_flop, dom_ms, dom_tr = "sdpa_kernel<128> S=4608 H=24", flop_sdpa, ms["sdpa_S4608"], "sdpa"
     else:
-        dom, dom_flop, dom_ms, dom_tr = ("dense_qx_kernel<6,256,256> M=4096 N=3x3072 K=3072 (fused norm/RoPE epilogue)",
-                                          2.0 * HW * C * 3 * C, ms["dense_qkv_image_M4096"], "dense_qkv_image")
+        dom, dom_flop, dom_ms, dom_tr = ("dense_qx_kernel<6,256,256> M=4096+512 N=3x3072 K=3072 (fused norm/RoPE epilogue)",
+                                          2.0 * S * C * 3 * C, ms["dense_qkv_grouped"], "dense_qkv_image")
     roofline = {
         "kernel": dom, "bound": "mfma", "achieved": round(tf(dom_flop, dom_ms), 2), "peak": PEAK_F16_TFLOPS,
         "unit": "TFLOP/s", "frac": round(tf(dom_flop, dom_ms) / PEAK_F16_TFLOPS, 4),

@@ -32,6 +32,7 @@ ABI_SYMBOLS = (
     "dt_depalettize_f16",
     "dt_dense_qx_f16",
     "dt_dense_qx_heads_f16",
+    "dt_dense_qx_grouped_f16",
     "dt_qk_norm_rope_f16",
     "dt_sdpa_f16",
     "dt_sdpa_workspace_bytes",
@@ -56,6 +57,12 @@ class _View4(ctypes.Structure):
 class _HeadEpilogue(ctypes.Structure):
     _fields_ = [("gamma", ctypes.c_void_p), ("rot", ctypes.c_void_p), ("rot_pos0", ctypes.c_int64),
                 ("eps", ctypes.c_float), ("head_dim", ctypes.c_int32)]
+
+
+class _DenseGroup(ctypes.Structure):
+    _fields_ = [("M", ctypes.c_int64), ("K", ctypes.c_int64), ("X", ctypes.c_void_p), ("ldx", ctypes.c_int64),
+                ("W", ctypes.c_void_p), ("n_weights", ctypes.c_int32), ("bias", ctypes.c_void_p),
+                ("Y", ctypes.c_void_p), ("ldy", ctypes.c_void_p), ("epi", ctypes.c_void_p)]
 
 
 class _Segment(ctypes.Structure):
@@ -103,6 +110,8 @@ def lib():
                                             ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(i64),
                                             ctypes.POINTER(_HeadEpilogue), ctypes.c_uint32]
         L.dt_qk_norm_rope_f16.restype = i32
+        L.dt_dense_qx_grouped_f16.restype = i32
+        L.dt_dense_qx_grouped_f16.argtypes = [vp, i32, ctypes.POINTER(_DenseGroup), ctypes.c_uint32]
         L.dt_qk_norm_rope_f16.argtypes = [vp, _View4, i32, i64, i32, i32, vp, f32, i32, vp, i64, f32]
         L.dt_sdpa_f16.restype = i32
         L.dt_sdpa_f16.argtypes = [vp, i32, i32, i32, i32, i32, ctypes.POINTER(_Segment), i32,
@@ -271,10 +280,8 @@ class HeadEpilogue:
     head_dim: int = 128
 
 
-def dense_multi(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]], outs=None, flags: int = 0,
-                stream=None, epilogues: Optional[Sequence[Optional[HeadEpilogue]]] = None):
-    """Several Dense ops that share the input, one launch (x_q / x_k / x_v).  `epilogues[i]` (optional) fuses the
-    per-head RMSNorm / RoPE that follows projection i."""
+def _marshal_dense(x, weights, biases, outs, epilogues):
+    """ctypes arguments of one Dense problem; returns (keepalive, fields, outs, M, x2)."""
     torch = _torch()
     _f16_cuda(x, "x")
     K = x.shape[-1]
@@ -293,10 +300,8 @@ def dense_multi(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object
     B = (vp * n)(*[None if b is None else _f16_cuda(b, "bias").data_ptr() for b in biases])
     Y = (vp * n)(*[o.data_ptr() for o in outs])
     LDY = (ctypes.c_int64 * n)(*[o.stride(0) for o in outs])
-    if epilogues is None:
-        st = lib().dt_dense_qx_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, flags)
-        _check("dt_dense_qx_f16", st)
-    else:
+    E = None
+    if epilogues is not None:
         E = (_HeadEpilogue * n)()
         for i, e in enumerate(epilogues):
             if e is None:
@@ -311,10 +316,40 @@ def dense_multi(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object
                 raise ValueError("gamma must hold head_dim elements")
             E[i] = _HeadEpilogue(None if e.gamma is None else e.gamma.data_ptr(),
                                  None if e.rot is None else e.rot.data_ptr(), e.rot_pos0, e.eps, e.head_dim)
-        st = lib().dt_dense_qx_heads_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, E, flags)
-        _check("dt_dense_qx_heads_f16", st)
+    return (x2, M, K, n, W, B, Y, LDY, E, outs)
+
+
+def _shape_outs(x, M, outs):
     lead = tuple(x.shape[:-1])
     return [o.reshape(lead + (o.shape[-1],)) if o.shape[0] == M and o.is_contiguous() else o for o in outs]
+
+
+def dense_multi(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]], outs=None, flags: int = 0,
+                stream=None, epilogues: Optional[Sequence[Optional[HeadEpilogue]]] = None):
+    """Several Dense ops that share the input, one launch (x_q / x_k / x_v).  `epilogues[i]` (optional) fuses the
+    per-head RMSNorm / RoPE that follows projection i."""
+    x2, M, K, n, W, B, Y, LDY, E, outs = _marshal_dense(x, weights, biases, outs, epilogues)
+    if E is None:
+        st = lib().dt_dense_qx_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, flags)
+        _check("dt_dense_qx_f16", st)
+    else:
+        st = lib().dt_dense_qx_heads_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, E, flags)
+        _check("dt_dense_qx_heads_f16", st)
+    return _shape_outs(x, M, outs)
+
+
+def dense_grouped(problems: Sequence[dict], flags: int = 0, stream=None):
+    """Independent Dense problems enqueued together (the context and image projections of a joint block).  Each
+    problem is a dict with the arguments of dense_multi: x, weights, biases, and optionally outs, epilogues.
+    Returns one list of outputs per problem."""
+    keep = [_marshal_dense(p["x"], p["weights"], p["biases"], p.get("outs"), p.get("epilogues")) for p in problems]
+    G = (_DenseGroup * len(keep))()
+    cast = lambda a: None if a is None else ctypes.addressof(a)  # the arrays stay alive in `keep` until the call returns
+    for i, (x2, M, K, n, W, B, Y, LDY, E, outs) in enumerate(keep):
+        G[i] = _DenseGroup(M, K, x2.data_ptr(), x2.stride(0), cast(W), n, cast(B), cast(Y), cast(LDY), cast(E))
+    st = lib().dt_dense_qx_grouped_f16(_stream_ptr(stream), len(keep), G, flags)
+    _check("dt_dense_qx_grouped_f16", st)
+    return [_shape_outs(p["x"], k[1], k[9]) for p, k in zip(problems, keep)]
 
 
 class Dense:

@@ -18,7 +18,8 @@
 
 namespace dt {
 
-constexpr int kMaxWeights = 4;
+constexpr int kMaxWeights = 8;
+constexpr int kMaxGroups = 4;
 constexpr int BK = 32;
 constexpr int LDS_ROW = BK + 8;  // halfs; 80-byte rows keep 16-byte LDS accesses of 8 consecutive rows on distinct banks
 constexpr int kPalLdsBytes = 32768;
@@ -44,14 +45,24 @@ struct DenseWeight {
   float eps;
 };
 
-struct DenseArgs {
+// One X with the weights applied to it; a launch runs up to kMaxGroups of them
+// (same K and weight format), their tiles numbered one group after the other.
+struct DenseGroup {
   const uint16_t* x;
   int64_t ldx;
-  int32_t m, k;
+  int32_t m;
+  int32_t tiles_m, tiles_n;
+  int32_t tile_begin;    // first tile of this group in the launch
+  int32_t w_begin, w_end;  // its weights in DenseArgs::w
+};
+
+struct DenseArgs {
+  int32_t k;
   int32_t nib;
   int32_t pal_step;  // K-tiles between columns at which a row can enter a new palette block: gcd(K, nib) / 32
-  int32_t n_weights;
-  int32_t tiles_m, tiles_n;
+  int32_t n_groups;
+  int32_t total_tiles;
+  DenseGroup g[kMaxGroups];
   DenseWeight w[kMaxWeights];
 };
 
@@ -146,27 +157,33 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // run together on an XCD cover a compact 2-D block of tiles (8 x 4 at 32 CUs),
   // so every X and W panel slice is fetched into that XCD's L2 once per block
   // instead of once per tile column.
-  const int total = a.tiles_m * a.tiles_n;
+  const int total = a.total_tiles;
   int bid = blockIdx.x;
   {
     const int per = total / 8;
     if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
   }
+  int gi = 0;
+#pragma unroll
+  for (int i = 1; i < kMaxGroups; i++)
+    if (i < a.n_groups && bid >= a.g[i].tile_begin) gi = i;
+  const DenseGroup g = a.g[gi];
+  bid -= g.tile_begin;
   int tm, tn;
   {
     constexpr int GM = 8;
-    const int band_tiles = GM * a.tiles_n;
+    const int band_tiles = GM * g.tiles_n;
     const int band = bid / band_tiles;
     const int in_band = bid - band * band_tiles;
-    const int rows_in_band = (a.tiles_m - band * GM) < GM ? (a.tiles_m - band * GM) : GM;
+    const int rows_in_band = (g.tiles_m - band * GM) < GM ? (g.tiles_m - band * GM) : GM;
     tn = in_band / rows_in_band;
     tm = band * GM + (in_band - tn * rows_in_band);
   }
 
-  int wi = 0;
+  int wi = g.w_begin;
 #pragma unroll
   for (int i = 1; i < kMaxWeights; i++)
-    if (i < a.n_weights && tn >= a.w[i].tile_begin) wi = i;
+    if (i > g.w_begin && i < g.w_end && tn >= a.w[i].tile_begin) wi = i;
   const DenseWeight w = a.w[wi];
   const int n0 = (tn - w.tile_begin) * BN;
   const int m0 = tm * BM;
@@ -186,10 +203,10 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     const int row = 8 * (wave * AP + i) + (lane >> 3);
     const int c8 = pair_chunk(row, lane & 7);
     int gm = m0 + row;
-    if (gm >= a.m) gm = a.m - 1;
-    a_off[i] = (uint32_t)(((int64_t)gm * a.ldx + c8 * 8) * 2);
+    if (gm >= g.m) gm = g.m - 1;
+    a_off[i] = (uint32_t)(((int64_t)gm * g.ldx + c8 * 8) * 2);
   }
-  const char* xbase = reinterpret_cast<const char*>(a.x);
+  const char* xbase = reinterpret_cast<const char*>(g.x);
   const char* wbase = reinterpret_cast<const char*>(w.data);
 
   // weight row of this thread (two threads per row; each loads and unpacks one half of the row's granule)
@@ -335,7 +352,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       }
 #pragma unroll
       for (int j = 4 * p; j < 4 * p + 4; j++)
-        la[j] = pal_base | (own_index<Q, HW>(be, j) << (MODE == kPalRow ? 7 : 1));  // disjoint bits
+        la[j] = own_index_at<Q, HW, (MODE == kPalRow ? 7 : 1)>(be, j, pal_base);
     }
   };
   auto lookup = [&](int j) {
@@ -569,7 +586,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
 #pragma unroll
       for (int j = 0; j < TM; j++) {
         const int gm = m0 + wm * WM + j * 32 + l32;
-        const int gmc = gm < a.m ? gm : a.m - 1;
+        const int gmc = gm < g.m ? gm : g.m - 1;
         uint16_t* yrow = w.y + (int64_t)gmc * w.ldy;
         float y[TN][16];
         float ss = 0.f;
@@ -639,7 +656,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
               run[e] = r[0];
               run[2 + e] = r[1];
             }
-            if (gm < a.m) *reinterpret_cast<uint4_t*>(yrow + nh + i * 32 + 16 * gp + 8 * hi) = uint4_t{run[0], run[1], run[2], run[3]};
+            if (gm < g.m) *reinterpret_cast<uint4_t*>(yrow + nh + i * 32 + 16 * gp + 8 * hi) = uint4_t{run[0], run[1], run[2], run[3]};
           }
         }
       }
@@ -655,7 +672,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
 #pragma unroll
   for (int j = 0; j < TM; j++) {
     const int gm = m0 + wm * WM + j * 32 + l32;
-    uint16_t* yrow = w.y + (int64_t)(gm < a.m ? gm : 0) * w.ldy;
+    uint16_t* yrow = w.y + (int64_t)(gm < g.m ? gm : 0) * w.ldy;
 #pragma unroll
     for (int i = 0; i < TN; i++) {
       const int nb = n0 + wn * WN + i * 32;
@@ -693,7 +710,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
           run[2 + e] = r[1];  // low lanes: high lanes' 2gp   | high lanes: own group 2gp+1
         }
         const int nn = nb + 16 * gp + 8 * hi;
-        if (gm < a.m) {
+        if (gm < g.m) {
           if (nn + 7 < w.n && ((w.ldy & 7) == 0) && ((reinterpret_cast<uintptr_t>(w.y) & 15) == 0)) {
             *reinterpret_cast<uint4_t*>(yrow + nn) = uint4_t{run[0], run[1], run[2], run[3]};
           } else {
@@ -739,7 +756,7 @@ __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* _
 
 template <int Q, int BM, int BN>
 static dt_status launch_tiled(hipStream_t s, const DenseArgs& a, int mode) {
-  dim3 grid((unsigned)(a.tiles_m * a.tiles_n)), block(512);
+  dim3 grid((unsigned)a.total_tiles), block(512);
   switch (mode) {
     case kPalShared: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalShared>), grid, block, 0, s, a); break;
     case kPalRow:
@@ -763,7 +780,7 @@ static dt_status launch_tiled_q(hipStream_t s, const DenseArgs& a, int qbits, in
     case 7: return launch_tiled<7, BM, BN>(s, a, mode);
     case 8: return launch_tiled<8, BM, BN>(s, a, mode);
     case 16: {
-      dim3 grid((unsigned)(a.tiles_m * a.tiles_n)), block(512);
+      dim3 grid((unsigned)a.total_tiles), block(512);
       hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16>), grid, block, 0, s, a);
       return launch_status();
     }
@@ -783,6 +800,233 @@ static int choose_pal_mode(int qbits, int nib, int64_t K, int BN) {
 
 }  // namespace dt
 
+namespace dt {
+
+// One Dense problem as the entry points receive it.
+struct HostGroup {
+  int64_t M, K;
+  const uint16_t* X;
+  int64_t ldx;
+  const dt_qx_weight* W;
+  int32_t n_weights;
+  const uint16_t* const* bias;
+  uint16_t* const* Y;
+  const int64_t* ldy;
+  const dt_head_epilogue* epi;
+
+  bool wants_epi(int wi) const { return epi && (epi[wi].gamma || epi[wi].rot); }
+  // fused head epilogue: in the tiled kernel for 128-wide heads that start on a 16-byte aligned,
+  // 8-element-strided output; otherwise the Dense runs plain and the norm / rotation pass follows
+  bool fusable(int wi) const {
+    return epi[wi].head_dim == 128 && (ldy[wi] % 8 == 0) && ((reinterpret_cast<uintptr_t>(Y[wi]) & 15) == 0) &&
+           (!epi[wi].gamma || (reinterpret_cast<uintptr_t>(epi[wi].gamma) & 7) == 0) &&
+           (!epi[wi].rot || (reinterpret_cast<uintptr_t>(epi[wi].rot) & 7) == 0) &&
+           (!bias || !bias[wi] || (reinterpret_cast<uintptr_t>(bias[wi]) & 7) == 0);
+  }
+  bool x_ok() const {
+    return (K % (2 * BK) == 0) && (ldx % 8 == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
+  }
+  bool w_tiled(int wi) const {
+    const dt_qx_weight& w = W[wi];
+    return w.count / K > 0 && (reinterpret_cast<uintptr_t>(w.data) & 15) == 0 && (w.qbits == 16 || w.nib % 32 == 0);
+  }
+};
+
+static dt_status validate_group(const HostGroup& h) {
+  if (h.epi && h.n_weights > 0) {
+    for (int i = 0; i < h.n_weights; i++) {
+      const dt_head_epilogue& e = h.epi[i];
+      if (!e.gamma && !e.rot) continue;
+      if (e.head_dim <= 0 || e.head_dim % 2 != 0 || e.head_dim > 128) return DT_NO_KERNEL;
+      if (e.rot && e.rot_pos0 < 0) return DT_INVALID;
+      if (h.Y && h.ldy && h.M > 0 && ((h.ldy[i] & 1) || (reinterpret_cast<uintptr_t>(h.Y[i]) & 3))) return DT_INVALID;
+      if (e.rot && (reinterpret_cast<uintptr_t>(e.rot) & 3)) return DT_INVALID;
+      if (h.W && h.K > 0 && h.W[i].count >= 0 && (h.W[i].count / h.K) % e.head_dim != 0) return DT_INVALID;
+    }
+  }
+  if (h.M < 0 || h.K <= 0 || h.n_weights <= 0 || !h.W || !h.Y || !h.ldy) return DT_INVALID;
+  if (h.M > 0x7fffffff || h.K > 0x7fffffff) return DT_INVALID;
+  for (int i = 0; i < h.n_weights; i++) {
+    const dt_qx_weight& w = h.W[i];
+    if (!w.data || w.count < 0 || w.count % h.K != 0) return DT_INVALID;
+    if (w.qbits != 16 && (w.qbits < 4 || w.qbits > 8 || w.nib <= 0)) return DT_INVALID;
+    if (w.count / h.K > 0x7fffffff) return DT_INVALID;
+    if (h.M > 0 && (!h.Y[i] || h.ldy[i] < w.count / h.K)) return DT_INVALID;
+  }
+  if (h.M > 0 && (!h.X || h.ldx < h.K)) return DT_INVALID;
+  return DT_OK;
+}
+
+static dt_status epilogue_pass(hipStream_t s, const HostGroup& h, int wi) {
+  QkPrepArgs p;
+  p.src = h.Y[wi];
+  p.dst = h.Y[wi];
+  p.src_sb = p.dst_sb = 0;
+  p.src_ss = p.dst_ss = h.ldy[wi];
+  p.src_sh = p.dst_sh = h.epi[wi].head_dim;
+  p.B = 1;
+  p.S = h.M;
+  p.H = (int32_t)((h.W[wi].count / h.K) / h.epi[wi].head_dim);
+  p.D = h.epi[wi].head_dim;
+  p.gamma = h.epi[wi].gamma;
+  p.eps = h.epi[wi].eps;
+  p.norm_per_head = 1;
+  p.rot = h.epi[wi].rot;
+  p.rot_pos0 = h.epi[wi].rot_pos0;
+  p.post_scale = 1.0f;
+  return qk_prep_launch(s, p);
+}
+
+// Appends weight wi of h to the launch; returns its number of N-tiles.
+static int add_weight(DenseArgs& a, int slot, const HostGroup& h, int wi, int tile_begin, int BN, bool fuse) {
+  const int64_t n_rows = h.W[wi].count / h.K;
+  DenseWeight& d = a.w[slot];
+  d.data = static_cast<const uint8_t*>(h.W[wi].data);
+  d.bias = h.bias ? h.bias[wi] : nullptr;
+  d.y = h.Y[wi];
+  d.ldy = h.ldy[wi];
+  d.n = (int32_t)n_rows;
+  d.tile_begin = tile_begin;
+  d.gamma = fuse ? h.epi[wi].gamma : nullptr;
+  d.rot = fuse ? h.epi[wi].rot : nullptr;
+  d.rot_pos0 = fuse ? h.epi[wi].rot_pos0 : 0;
+  d.eps = fuse ? h.epi[wi].eps : 0.f;
+  return (int)((n_rows + BN - 1) / BN);
+}
+
+static void finish_args(DenseArgs& a, int n_groups, int n_w, int64_t K, const dt_qx_weight& w0) {
+  for (int j = n_w; j < kMaxWeights; j++) a.w[j] = a.w[0];
+  for (int j = n_groups; j < kMaxGroups; j++) a.g[j] = a.g[0];
+  a.n_groups = n_groups;
+  a.k = (int32_t)K;
+  a.nib = w0.qbits == 16 ? 32 : w0.nib;
+  a.pal_step = (int32_t)(std::gcd((int64_t)K, (int64_t)a.nib) / BK);
+}
+
+// One validated problem with M > 0: weights that share (qbits, nib) and meet the
+// tiled kernel's alignment go out in runs of up to kMaxWeights per launch; the
+// rest take the generic kernel.
+static dt_status run_group(hipStream_t s, const HostGroup& h) {
+  const int64_t M = h.M, K = h.K;
+  const bool x_ok = h.x_ok();
+  int i = 0;
+  while (i < h.n_weights) {
+    const dt_qx_weight& w0 = h.W[i];
+    const int64_t n_rows0 = w0.count / K;
+    if (!(x_ok && h.w_tiled(i))) {
+      if (n_rows0 > 0) {
+        int64_t outs = M * n_rows0;
+        if ((outs + 255) / 256 > 0x7fffffff) return DT_NO_KERNEL;
+        hipLaunchKernelGGL(dense_qx_generic_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, s, h.X, h.ldx,
+                           M, n_rows0, K, static_cast<const uint8_t*>(w0.data), w0.qbits, w0.nib,
+                           h.bias ? h.bias[i] : nullptr, h.Y[i], h.ldy[i]);
+        dt_status st = launch_status();
+        if (st != DT_OK) return st;
+        if (h.wants_epi(i)) {
+          st = epilogue_pass(s, h, i);
+          if (st != DT_OK) return st;
+        }
+      }
+      i++;
+      continue;
+    }
+    // tile shape: big tiles when there is enough work to fill 256 CUs with them
+    bool any_fused = false;
+    for (int j = i; j < h.n_weights && j < i + kMaxWeights; j++)
+      any_fused = any_fused || (h.wants_epi(j) && h.fusable(j));
+    const bool big = ((M >= 1024) && (n_rows0 >= 256)) || any_fused;  // the fused epilogue needs the 128-feature wave slice
+    // few token rows: halve the token tile so that more workgroups share the work
+    const bool narrow = big && M < 1024;
+    const int BM = big ? (narrow ? 128 : 256) : 128, BN = big ? 256 : 128;
+    DenseArgs a;
+    DenseGroup& g = a.g[0];
+    g.x = h.X;
+    g.ldx = h.ldx;
+    g.m = (int32_t)M;
+    g.tiles_m = (int)((M + BM - 1) / BM);
+    g.tile_begin = 0;
+    g.w_begin = 0;
+    int tiles_n = 0, cnt = 0;
+    const int first = i;
+    while (i < h.n_weights && cnt < kMaxWeights) {
+      const dt_qx_weight& w = h.W[i];
+      if (w.qbits != w0.qbits || (w.qbits != 16 && w.nib != w0.nib) || !h.w_tiled(i)) break;
+      tiles_n += add_weight(a, cnt, h, i, tiles_n, BN, big && h.wants_epi(i) && h.fusable(i));
+      cnt++;
+      i++;
+    }
+    g.w_end = cnt;
+    g.tiles_n = tiles_n;
+    if ((int64_t)g.tiles_m * tiles_n > 0x7fffffff) return DT_NO_KERNEL;
+    a.total_tiles = g.tiles_m * tiles_n;
+    finish_args(a, 1, cnt, K, w0);
+    const int mode = choose_pal_mode(w0.qbits, a.nib, K, BN);
+    dt_status st = !big ? launch_tiled_q<128, 128>(s, a, w0.qbits, mode)
+                   : narrow ? launch_tiled_q<128, 256>(s, a, w0.qbits, mode)
+                            : launch_tiled_q<256, 256>(s, a, w0.qbits, mode);
+    if (st != DT_OK) return st;
+    for (int j = first; j < i; j++)
+      if (h.wants_epi(j) && !(big && h.fusable(j))) {
+        st = epilogue_pass(s, h, j);
+        if (st != DT_OK) return st;
+      }
+  }
+  return DT_OK;
+}
+
+// All problems in one launch of 256 x 256 tiles, when every X and weight meets
+// the tiled kernel's alignment, they share K and the weight format, and at least
+// one of them is large enough for that tile.  Returns false if they do not fit.
+static bool run_groups_fused(hipStream_t s, const HostGroup* hs, int n, dt_status* status) {
+  if (n < 2 || n > kMaxGroups) return false;
+  const dt_qx_weight& w0 = hs[0].W[0];
+  int total_w = 0;
+  bool big = false;
+  for (int gi = 0; gi < n; gi++) {
+    const HostGroup& h = hs[gi];
+    if (h.K != hs[0].K || !h.x_ok()) return false;
+    for (int i = 0; i < h.n_weights; i++) {
+      const dt_qx_weight& w = h.W[i];
+      if (!h.w_tiled(i) || w.qbits != w0.qbits || (w.qbits != 16 && w.nib != w0.nib)) return false;
+      big = big || (h.M >= 1024 && w.count / h.K >= 256);
+    }
+    total_w += h.n_weights;
+  }
+  if (!big || total_w > kMaxWeights) return false;
+  constexpr int BM = 256, BN = 256;
+  DenseArgs a;
+  int cnt = 0;
+  int64_t tiles = 0;
+  for (int gi = 0; gi < n; gi++) {
+    const HostGroup& h = hs[gi];
+    DenseGroup& g = a.g[gi];
+    g.x = h.X;
+    g.ldx = h.ldx;
+    g.m = (int32_t)h.M;
+    g.tiles_m = (int)((h.M + BM - 1) / BM);
+    g.tile_begin = (int32_t)tiles;
+    g.w_begin = cnt;
+    int tiles_n = 0;
+    for (int i = 0; i < h.n_weights; i++, cnt++)
+      tiles_n += add_weight(a, cnt, h, i, tiles_n, BN, h.wants_epi(i) && h.fusable(i));
+    g.w_end = cnt;
+    g.tiles_n = tiles_n;
+    tiles += (int64_t)g.tiles_m * tiles_n;
+    if (tiles > 0x7fffffff) return false;
+  }
+  a.total_tiles = (int32_t)tiles;
+  finish_args(a, n, cnt, hs[0].K, w0);
+  const int mode = choose_pal_mode(w0.qbits, a.nib, hs[0].K, BN);
+  dt_status st = launch_tiled_q<BM, BN>(s, a, w0.qbits, mode);
+  for (int gi = 0; gi < n && st == DT_OK; gi++)
+    for (int i = 0; i < hs[gi].n_weights && st == DT_OK; i++)
+      if (hs[gi].wants_epi(i) && !hs[gi].fusable(i)) st = epilogue_pass(s, hs[gi], i);
+  *status = st;
+  return true;
+}
+
+}  // namespace dt
+
 DT_EXPORT dt_status dt_dense_qx_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,
                                     const dt_qx_weight* W, int32_t n_weights, const uint16_t* const* bias,
                                     uint16_t* const* Y, const int64_t* ldy, uint32_t flags) {
@@ -795,136 +1039,37 @@ DT_EXPORT dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K
                                           uint32_t flags) {
   using namespace dt;
   (void)flags;
-  if (epi && n_weights > 0) {
-    for (int i = 0; i < n_weights; i++) {
-      if (!epi[i].gamma && !epi[i].rot) continue;
-      if (epi[i].head_dim <= 0 || epi[i].head_dim % 2 != 0 || epi[i].head_dim > 128) return DT_NO_KERNEL;
-      if (epi[i].rot && epi[i].rot_pos0 < 0) return DT_INVALID;
-      if (Y && ldy && M > 0 && ((ldy[i] & 1) || (reinterpret_cast<uintptr_t>(Y[i]) & 3))) return DT_INVALID;
-      if (epi[i].rot && (reinterpret_cast<uintptr_t>(epi[i].rot) & 3)) return DT_INVALID;
-      if (W && K > 0 && W[i].count >= 0 && (W[i].count / K) % epi[i].head_dim != 0) return DT_INVALID;
-    }
-  }
-  if (M < 0 || K <= 0 || n_weights <= 0 || !W || !Y || !ldy) return DT_INVALID;
-  if (M > 0x7fffffff || K > 0x7fffffff) return DT_INVALID;
-  for (int i = 0; i < n_weights; i++) {
-    const dt_qx_weight& w = W[i];
-    if (!w.data || w.count < 0 || w.count % K != 0) return DT_INVALID;
-    if (w.qbits != 16 && (w.qbits < 4 || w.qbits > 8 || w.nib <= 0)) return DT_INVALID;
-    if (w.count / K > 0x7fffffff) return DT_INVALID;
-    if (M > 0 && (!Y[i] || ldy[i] < w.count / K)) return DT_INVALID;
-  }
+  const HostGroup h{M, K, X, ldx, W, n_weights, bias, Y, ldy, epi};
+  dt_status st = validate_group(h);
+  if (st != DT_OK) return st;
   if (M == 0) return DT_OK;
-  if (!X || ldx < K) return DT_INVALID;
+  if (!device_ok()) return DT_NO_KERNEL;
+  return run_group(as_stream(stream), h);
+}
+
+DT_EXPORT dt_status dt_dense_qx_grouped_f16(dt_stream stream, int32_t n_groups, const dt_dense_group* groups,
+                                            uint32_t flags) {
+  using namespace dt;
+  (void)flags;
+  if (n_groups < 0 || (n_groups > 0 && !groups)) return DT_INVALID;
+  if (n_groups > 64) return DT_INVALID;
+  HostGroup hs[64];
+  int n = 0;
+  for (int i = 0; i < n_groups; i++) {
+    const dt_dense_group& d = groups[i];
+    const HostGroup h{d.M, d.K, d.X, d.ldx, d.W, d.n_weights, d.bias, d.Y, d.ldy, d.epi};
+    dt_status st = validate_group(h);
+    if (st != DT_OK) return st;
+    if (h.M > 0) hs[n++] = h;
+  }
+  if (n == 0) return DT_OK;
   if (!device_ok()) return DT_NO_KERNEL;
   hipStream_t s = as_stream(stream);
-
-  // Weights that share (qbits, nib) and meet the tiled kernel's alignment go
-  // out in groups of up to kMaxWeights per launch; the rest take the generic kernel.
-  const bool x_ok = (K % (2 * BK) == 0) && (ldx % 8 == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
-  int i = 0;
-  while (i < n_weights) {
-    const dt_qx_weight& w0 = W[i];
-    const int64_t n_rows0 = w0.count / K;
-    bool tiled = x_ok && n_rows0 > 0 && (reinterpret_cast<uintptr_t>(w0.data) & 15) == 0 &&
-                 (w0.qbits == 16 || w0.nib % 32 == 0);
-    // fused head epilogue: in the tiled kernel for 128-wide heads that start on a 16-byte aligned,
-    // 8-element-strided output; otherwise the Dense runs plain and the norm / rotation pass follows
-    auto wants_epi = [&](int wi) { return epi && (epi[wi].gamma || epi[wi].rot); };
-    auto fusable = [&](int wi) {
-      return epi[wi].head_dim == 128 && (ldy[wi] % 8 == 0) && ((reinterpret_cast<uintptr_t>(Y[wi]) & 15) == 0) &&
-             (!epi[wi].gamma || (reinterpret_cast<uintptr_t>(epi[wi].gamma) & 7) == 0) &&
-             (!epi[wi].rot || (reinterpret_cast<uintptr_t>(epi[wi].rot) & 7) == 0) &&
-             (!bias || !bias[wi] || (reinterpret_cast<uintptr_t>(bias[wi]) & 7) == 0);
-    };
-    auto epilogue_pass = [&](int wi) -> dt_status {
-      QkPrepArgs p;
-      p.src = Y[wi];
-      p.dst = Y[wi];
-      p.src_sb = p.dst_sb = 0;
-      p.src_ss = p.dst_ss = ldy[wi];
-      p.src_sh = p.dst_sh = epi[wi].head_dim;
-      p.B = 1;
-      p.S = M;
-      p.H = (int32_t)((W[wi].count / K) / epi[wi].head_dim);
-      p.D = epi[wi].head_dim;
-      p.gamma = epi[wi].gamma;
-      p.eps = epi[wi].eps;
-      p.norm_per_head = 1;
-      p.rot = epi[wi].rot;
-      p.rot_pos0 = epi[wi].rot_pos0;
-      p.post_scale = 1.0f;
-      return qk_prep_launch(s, p);
-    };
-    if (!tiled) {
-      if (n_rows0 > 0) {
-        int64_t outs = M * n_rows0;
-        if ((outs + 255) / 256 > 0x7fffffff) return DT_NO_KERNEL;
-        hipLaunchKernelGGL(dense_qx_generic_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, s, X, ldx, M,
-                           n_rows0, K, static_cast<const uint8_t*>(w0.data), w0.qbits, w0.nib,
-                           bias ? bias[i] : nullptr, Y[i], ldy[i]);
-        dt_status st = launch_status();
-        if (st != DT_OK) return st;
-        if (wants_epi(i)) {
-          st = epilogue_pass(i);
-          if (st != DT_OK) return st;
-        }
-      }
-      i++;
-      continue;
-    }
-    // tile shape: big tiles when there is enough work to fill 256 CUs with them
-    bool any_fused = false;
-    for (int j = i; j < n_weights && j < i + kMaxWeights; j++) any_fused = any_fused || (wants_epi(j) && fusable(j));
-    const bool big = ((M >= 1024) && (n_rows0 >= 256)) || any_fused;  // the fused epilogue needs the 128-feature wave slice
-    // few token rows: halve the token tile so that more workgroups share the work
-    const bool narrow = big && M < 1024;
-    const int BM = big ? (narrow ? 128 : 256) : 128, BN = big ? 256 : 128;
-    DenseArgs a;
-    a.x = X;
-    a.ldx = ldx;
-    a.m = (int32_t)M;
-    a.k = (int32_t)K;
-    a.nib = w0.qbits == 16 ? 32 : w0.nib;
-    a.pal_step = (int32_t)(std::gcd((int64_t)K, (int64_t)a.nib) / BK);
-    a.tiles_m = (int)((M + BM - 1) / BM);
-    int tiles_n = 0, cnt = 0;
-    const int first = i;
-    while (i < n_weights && cnt < kMaxWeights) {
-      const dt_qx_weight& w = W[i];
-      const int64_t n_rows = w.count / K;
-      if (w.qbits != w0.qbits || (w.qbits != 16 && w.nib != w0.nib) || n_rows <= 0 ||
-          (reinterpret_cast<uintptr_t>(w.data) & 15) != 0)
-        break;
-      a.w[cnt].data = static_cast<const uint8_t*>(w.data);
-      a.w[cnt].bias = bias ? bias[i] : nullptr;
-      a.w[cnt].y = Y[i];
-      a.w[cnt].ldy = ldy[i];
-      a.w[cnt].n = (int32_t)n_rows;
-      a.w[cnt].tile_begin = tiles_n;
-      const bool fuse = big && wants_epi(i) && fusable(i);
-      a.w[cnt].gamma = fuse ? epi[i].gamma : nullptr;
-      a.w[cnt].rot = fuse ? epi[i].rot : nullptr;
-      a.w[cnt].rot_pos0 = fuse ? epi[i].rot_pos0 : 0;
-      a.w[cnt].eps = fuse ? epi[i].eps : 0.f;
-      tiles_n += (int)((n_rows + BN - 1) / BN);
-      cnt++;
-      i++;
-    }
-    for (int j = cnt; j < kMaxWeights; j++) a.w[j] = a.w[0];
-    a.n_weights = cnt;
-    a.tiles_n = tiles_n;
-    if ((int64_t)a.tiles_m * tiles_n > 0x7fffffff) return DT_NO_KERNEL;
-    const int mode = choose_pal_mode(w0.qbits, a.nib, K, BN);
-    dt_status st = !big ? launch_tiled_q<128, 128>(s, a, w0.qbits, mode)
-                   : narrow ? launch_tiled_q<128, 256>(s, a, w0.qbits, mode)
-                            : launch_tiled_q<256, 256>(s, a, w0.qbits, mode);
+  dt_status st = DT_OK;
+  if (run_groups_fused(s, hs, n, &st)) return st;
+  for (int i = 0; i < n; i++) {
+    st = run_group(s, hs[i]);
     if (st != DT_OK) return st;
-    for (int j = first; j < i; j++)
-      if (wants_epi(j) && !(big && fusable(j))) {
-        st = epilogue_pass(j);
-        if (st != DT_OK) return st;
-      }
   }
   return DT_OK;
 }

@@ -126,6 +126,26 @@ __device__ __forceinline__ void own_bits(const uint32_t (&own)[HW], bool upper, 
     for (int i = 0; i < HW; i++) be[i] = upper ? __builtin_amdgcn_alignbit(be[i], be[i + 1], 16) : be[i];
   }
 }
+// own_index() << SH | base in two instructions (shift or funnel shift, then
+// v_and_or_b32); base must have no bit in common with the shifted index.
+template <int Q, int HW, int SH>
+__device__ __forceinline__ uint32_t own_index_at(const uint32_t (&be)[HW + 1], int j, uint32_t base) {
+  const int bit = j * Q;
+  const int word = bit >> 5;
+  const int off = bit & 31;
+  const uint32_t mask = ((1u << Q) - 1) << SH;
+  uint32_t v;
+  if (off + Q <= 32) {
+    const int r = 32 - off - Q - SH;  // right shift that leaves the index at bit SH
+    v = r >= 0 ? be[word] >> r : be[word] << -r;
+  } else {
+    const int r = 64 - off - Q - SH;  // > 0: the index straddles two dwords
+    v = r < 32 ? __builtin_amdgcn_alignbit(be[word], be[word + 1], r) : be[word] >> (r - 32);
+  }
+  uint32_t out;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(out) : "v"(v), "s"(mask), "v"(base));
+  return out;
+}
 template <int Q, int HW>
 __device__ __forceinline__ uint32_t own_index(const uint32_t (&be)[HW + 1], int j) {
   const int bit = j * Q;

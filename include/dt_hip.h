@@ -150,6 +150,33 @@ dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K, const ui
                                 uint32_t flags);
 
 /*
+ * Several independent Dense problems (each an X with its weights, arguments as
+ * for dt_dense_qx_heads_f16) enqueued together.  The context (text) and image
+ * streams of a joint block apply different weights to different token sets
+ * (c_q / c_k / c_v and x_q / x_k / x_v, Models/Flux1.swift:161-176; c_o and
+ * x_o, 237-245); run as one launch the short text problem fills the compute
+ * units that the image problem's last round of tiles leaves idle.  Problems
+ * that share K and the weight format and meet the alignment of the tiled
+ * kernel go out in a single launch; anything else runs problem by problem with
+ * the same results.  Outputs of different problems must not overlap.
+ * `groups` is a HOST array.
+ */
+typedef struct {
+  int64_t M, K;
+  const uint16_t* X;
+  int64_t ldx;
+  const dt_qx_weight* W;
+  int32_t n_weights;
+  const uint16_t* const* bias;
+  uint16_t* const* Y;
+  const int64_t* ldy;
+  const dt_head_epilogue* epi;
+} dt_dense_group;
+
+dt_status dt_dense_qx_grouped_f16(dt_stream stream, int32_t n_groups, const dt_dense_group* groups,
+                                  uint32_t flags);
+
+/*
  * In place on a [B, S, H, D] view: optional RMSNorm, then optional RoPE.
  *   gamma       : RMSNorm weight, [D] when norm_per_head != 0 (Flux:
  *                 RMSNorm(axis: [3]), Models/Flux1.swift:165), [H*D] when 0

@@ -247,3 +247,59 @@ def test_dense_fused_head_norm_rope(dthip, oracle, torch_cuda, M, head_dim, q, n
         y = oracle.C.rmsnorm(y, gammas[0], 1e-6) if epi1.rot is None else oracle.C.cmul(y, rot[pos0:])
         mx, rr = oracle.err_stats(o1, y.reshape(M, N))
         assert mx <= MAX_ABS and rr <= 2 * REL_RMS, (mx, rr)
+
+
+@pytest.mark.parametrize("Ms,q,nib", [((1100, 200), 6, 4096), ((1030, 70, 300), 4, 512), ((200, 90), 6, 4096), ((1024, 256), 16, 0)])
+def test_dense_grouped_equals_separate(dthip, oracle, torch_cuda, Ms, q, nib):
+    """Independent problems (different X, weights, epilogues) enqueued as one call give bit-identical results to
+    one dt_dense call per problem, and both match the oracle.  The first two cases go out as a single launch
+    (a problem with >= 1024 rows), the third falls back to problem-by-problem."""
+    torch = torch_cuda
+    rng = np.random.default_rng(sum(Ms) + q)
+    K, H, hd = 256, 2, 128
+    N = H * hd
+    problems, packs, Xs, gam = [], [], [], []
+    for gi, M in enumerate(Ms):
+        X = rng.standard_normal((M, K)).astype(np.float16)
+        Xs.append(X)
+        ws, ps = [], []
+        for i in range(2):
+            if q == 16:
+                Wh = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+                ws.append(dthip.QxTensor.from_f16(Wh))
+                ps.append(Wh)
+            else:
+                w, p = make_weight(dthip, oracle, rng, N, K, q, nib, std=0.05)
+                ws.append(w)
+                ps.append(p)
+        packs.append(ps)
+        g = (1 + 0.05 * rng.standard_normal(hd)).astype(np.float16)
+        gam.append(g)
+        epi = [dthip.HeadEpilogue(to_dev(torch, g), None, 0, 1e-6, hd), None] if gi != 1 else None
+        problems.append(dict(x=to_dev(torch, X), weights=ws, biases=[None, None], epilogues=epi))
+    print("dense grouped", Ms, q, flush=True)
+    together = dthip.dense_grouped(problems)
+    for gi, p in enumerate(problems):
+        alone = dthip.dense_multi(p["x"], p["weights"], p["biases"], epilogues=p["epilogues"])
+        for i in range(2):
+            assert torch.equal(together[gi][i], alone[i]), (gi, i)
+            ref = oracle.C.dense(Xs[gi], packs[gi][i]) if q == 16 else oracle.C.dense_qx(Xs[gi], packs[gi][i], q, nib, N)
+            if p["epilogues"] is not None and i == 0:
+                ref = oracle.C.rmsnorm(ref.reshape(-1, H, hd), gam[gi], 1e-6).reshape(-1, N)
+            mx, rr = oracle.err_stats(together[gi][i].cpu().numpy(), ref)
+            assert mx <= MAX_ABS and rr <= 2 * REL_RMS, (gi, i, mx, rr)
+
+
+def test_dense_grouped_empty_and_bad(dthip, oracle, torch_cuda):
+    torch = torch_cuda
+    rng = np.random.default_rng(5)
+    assert dthip.dense_grouped([]) == []
+    w, _ = make_weight(dthip, oracle, rng, 64, 64, 6, 64)
+    x0 = torch.zeros((0, 64), dtype=torch.float16, device="cuda")
+    x1 = to_dev(torch, rng.standard_normal((5, 64)).astype(np.float16))
+    outs = dthip.dense_grouped([dict(x=x0, weights=[w], biases=[None]), dict(x=x1, weights=[w], biases=[None])])
+    assert outs[0][0].shape == (0, 64) and outs[1][0].shape == (5, 64)
+    assert torch.equal(outs[1][0], dthip.dense_multi(x1, [w], [None])[0])
+    bad = dthip.QxTensor(w.data, 3, w.nib, w.shape)
+    with pytest.raises(dthip.DtError):
+        dthip.dense_grouped([dict(x=x1, weights=[w], biases=[None]), dict(x=x1, weights=[bad], biases=[None])])
