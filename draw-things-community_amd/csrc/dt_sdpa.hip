@@ -28,6 +28,13 @@ constexpr int QROWS = QWAVES * 32;
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// One wave-wide memory -> LDS transfer: an active lane l's 16 bytes at g land
+// at LDS address lds + 16 * l (lds wave-uniform).
+__device__ __forceinline__ void load_to_lds_16(const void* g, unsigned char* lds) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                   (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+}
 // LDS layouts (measured bank-conflict free on this part: 64 banks, 16 lanes of
 // a 16-byte access or 32 lanes of an 8-byte access per clock).
 // K tile: [64 keys][DP] halfs; 16-byte chunk c of key row r is stored at a
@@ -47,7 +54,7 @@ __device__ __forceinline__ int v_unit_swz(int row, int u) {
   return u ^ ((row >> 1) & 1);
 }
 
-template <int DP, bool PREMUL>
+template <int DP, bool PREMUL, bool ONESEG>
 __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   constexpr int ROWB = DP * 2;                 // bytes per tile row
   constexpr int DCH = DP / 8;                  // 16-byte chunks per row
@@ -57,7 +64,13 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   constexpr int KS = DP / 16;                  // MFMA k-steps over the head dimension
   static_assert(LOADS >= 1, "tile");
 
-  __shared__ __attribute__((aligned(16))) unsigned char smem[4 * TILE_B];  // K stage 0, K stage 1, V stage 0, V stage 1
+  // Two stages each for K and V, as separate arrays: a tile is read from one
+  // while the next is in flight into the other, and only for distinct arrays
+  // does the compiler know that those reads need not wait for the transfer.
+  __shared__ __attribute__((aligned(1024))) unsigned char Ks0[TILE_B];
+  __shared__ __attribute__((aligned(1024))) unsigned char Ks1[TILE_B];
+  __shared__ __attribute__((aligned(1024))) unsigned char Vs0[TILE_B];
+  __shared__ __attribute__((aligned(1024))) unsigned char Vs1[TILE_B];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -101,18 +114,22 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   }
 
   // ---- K / V tile loaders ------------------------------------------------
-  // Each thread moves LOADS 16-byte chunks of every K tile and of every V tile.
-  // Row pointers advance by 64 rows per tile; they are re-derived from the
-  // segment table only when a row leaves its segment.
-  int k_dst[LOADS], v_dst[LOADS], ld_row[LOADS], ld_ch[LOADS];
+  // Tiles go from memory straight into LDS.  A wave's transfer instruction
+  // fills 1 KB of a tile, lane l landing on its 16-byte slot l; each thread
+  // issues LOADS of them per K tile and per V tile and fetches the chunk that
+  // the swizzle assigns to its slot.  Lanes whose row lies past the last key,
+  // or whose chunk lies past D, stay idle: those slots keep what they held
+  // (zeros from the start, or an earlier tile's finite values), which the
+  // masked scores and the zero padding of Q make harmless.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  int ld_row[LOADS], k_ch[LOADS], v_ch[LOADS];
 #pragma unroll
   for (int i = 0; i < LOADS; i++) {
-    const int c = tid + i * 512;
-    const int row = c / DCH, ch = c % DCH;
+    const int off = (wave * LOADS + i) * 1024 + lane * 16;
+    const int row = off / ROWB, pc = (off % ROWB) / 16;
     ld_row[i] = row;
-    ld_ch[i] = ch;
-    k_dst[i] = row * ROWB + k_chunk_swz<DP>(row, ch) * 16;
-    v_dst[i] = row * ROWB + v_unit_swz<DP>(row, ch >> 2) * 64 + (ch & 3) * 16;
+    k_ch[i] = k_chunk_swz<DP>(row, pc);  // the swizzles are involutions
+    v_ch[i] = v_unit_swz<DP>(row, pc >> 2) * 4 + (pc & 3);
   }
   struct RowPtr {
     const uint16_t* p;  // chunk address of the current row
@@ -120,7 +137,7 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     int64_t end;        // first joint row past the current segment
     int64_t step;       // elements per 64 rows inside the current segment
   };
-  auto locate = [&](const SdpaSeg* segs, int64_t kj, int ch, RowPtr& r) {
+  auto locate = [&](const SdpaSeg* segs, int64_t kj, int ch, RowPtr& r) __attribute__((always_inline)) {
     int sg = 0;
 #pragma unroll
     for (int i = 1; i < kMaxSeg; i++)
@@ -130,8 +147,8 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     r.end = (sg + 1 < a.n_kvseg) ? segs[sg + 1].start : Skv;
     r.step = segs[sg].ss * BKV;
   };
-  const bool one_seg = a.n_kvseg == 1;
-  auto advance = [&](const SdpaSeg* segs, int ch, RowPtr& r) {
+  const bool one_seg = a.n_kvseg == 1;  // uniform
+  auto advance = [&](const SdpaSeg* segs, int ch, RowPtr& r) __attribute__((always_inline)) {
     const int64_t kj = r.row + BKV;
     if (one_seg) {  // uniform: rows past the end are never dereferenced
       r.row = kj;
@@ -145,44 +162,71 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       r.row = kj;
     }
   };
-  RowPtr kp[LOADS], vp[LOADS];
+  RowPtr kp[ONESEG ? 1 : LOADS], vp[ONESEG ? 1 : LOADS];
+  // ONESEG: K and V are one run of rows each and small enough for 32-bit byte
+  // offsets from a uniform base; a tile step adds a uniform stride.
+  uint32_t k_off[LOADS], v_off[LOADS];
+  const char* k_base = nullptr;
+  const char* v_base = nullptr;
+  uint32_t k_step = 0, v_step = 0;
+  int rows_left = (int)(Skv < 0x7fffffff ? Skv : 0x7fffffff);  // ONESEG: keys from the next K tile on
+  int rows_left_v = rows_left;
+  if constexpr (ONESEG) {
+    k_base = reinterpret_cast<const char*>(a.k[0].ptr + b * a.k[0].sb + hk * a.k[0].sh);
+    v_base = reinterpret_cast<const char*>(a.v[0].ptr + b * a.v[0].sb + hk * a.v[0].sh);
+    k_step = (uint32_t)(a.k[0].ss * BKV * 2);
+    v_step = (uint32_t)(a.v[0].ss * BKV * 2);
 #pragma unroll
-  for (int i = 0; i < LOADS; i++) {
-    locate(a.k, ld_row[i] < Skv ? ld_row[i] : 0, ld_ch[i], kp[i]);
-    kp[i].row = ld_row[i];
-    locate(a.v, ld_row[i] < Skv ? ld_row[i] : 0, ld_ch[i], vp[i]);
-    vp[i].row = ld_row[i];
+    for (int i = 0; i < LOADS; i++) {
+      k_off[i] = (uint32_t)((ld_row[i] * a.k[0].ss + k_ch[i] * 8) * 2);
+      v_off[i] = (uint32_t)((ld_row[i] * a.v[0].ss + v_ch[i] * 8) * 2);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < LOADS; i++) {
+      locate(a.k, ld_row[i] < Skv ? ld_row[i] : 0, k_ch[i], kp[i]);
+      kp[i].row = ld_row[i];
+      locate(a.v, ld_row[i] < Skv ? ld_row[i] : 0, v_ch[i], vp[i]);
+      vp[i].row = ld_row[i];
+    }
   }
-  uint4_t k_reg[LOADS], v_reg[LOADS];
-  // loads the K (or V) tile the pointers stand on, then moves them to the next tile
-  auto issue_k = [&]() {
+  // starts the transfer of the K (or V) tile the pointers stand on, then moves them to the next tile
+  auto issue_k = [&](unsigned char* dst) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
-      uint4_t kv = uint4_t{0, 0, 0, 0};
-      if (kp[i].row < Skv && ld_ch[i] * 8 < D) kv = *reinterpret_cast<const uint4_t*>(kp[i].p);
-      k_reg[i] = kv;
-      advance(a.k, ld_ch[i], kp[i]);
+      if constexpr (ONESEG) {
+        if (ld_row[i] < rows_left && k_ch[i] * 8 < D) load_to_lds_16(k_base + k_off[i], dst + (wave_u * LOADS + i) * 1024);
+        k_off[i] += k_step;
+      } else {
+        if (kp[i].row < Skv && k_ch[i] * 8 < D) load_to_lds_16(kp[i].p, dst + (wave_u * LOADS + i) * 1024);
+        advance(a.k, k_ch[i], kp[i]);
+      }
     }
+    rows_left -= BKV;
   };
-  auto issue_v = [&]() {
+  auto issue_v = [&](unsigned char* dst) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
-      uint4_t vv = uint4_t{0, 0, 0, 0};  // rows past the end must be zero: 0 * garbage could be NaN
-      if (vp[i].row < Skv && ld_ch[i] * 8 < D) vv = *reinterpret_cast<const uint4_t*>(vp[i].p);
-      v_reg[i] = vv;
-      advance(a.v, ld_ch[i], vp[i]);
+      if constexpr (ONESEG) {
+        if (ld_row[i] < rows_left_v && v_ch[i] * 8 < D) load_to_lds_16(v_base + v_off[i], dst + (wave_u * LOADS + i) * 1024);
+        v_off[i] += v_step;
+      } else {
+        if (vp[i].row < Skv && v_ch[i] * 8 < D) load_to_lds_16(vp[i].p, dst + (wave_u * LOADS + i) * 1024);
+        advance(a.v, v_ch[i], vp[i]);
+      }
     }
+    rows_left_v -= BKV;
   };
-  auto stage_k = [&](int st) {
-    unsigned char* kb = smem + st * TILE_B;
-#pragma unroll
-    for (int i = 0; i < LOADS; i++) *reinterpret_cast<uint4_t*>(kb + k_dst[i]) = k_reg[i];
-  };
-  auto stage_v = [&](int st) {
-    unsigned char* vb = smem + (2 + st) * TILE_B;
-#pragma unroll
-    for (int i = 0; i < LOADS; i++) *reinterpret_cast<uint4_t*>(vb + v_dst[i]) = v_reg[i];
-  };
+  // slots that no transfer will ever write must not hold NaN patterns
+  if (D < DP || Skv % BKV != 0) {
+    for (int i = tid * 16; i < TILE_B; i += 512 * 16) {
+      *reinterpret_cast<uint4_t*>(Ks0 + i) = uint4_t{0, 0, 0, 0};
+      *reinterpret_cast<uint4_t*>(Ks1 + i) = uint4_t{0, 0, 0, 0};
+      *reinterpret_cast<uint4_t*>(Vs0 + i) = uint4_t{0, 0, 0, 0};
+      *reinterpret_cast<uint4_t*>(Vs1 + i) = uint4_t{0, 0, 0, 0};
+    }
+    __syncthreads();
+  }
 
   // ---- per-lane LDS read offsets --------------------------------------------
   // K operand: key row kb*32 + l32, chunk 2*ks + hi
@@ -217,15 +261,14 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   half8_t pf[2][2];    // its probabilities, as the B operand of the second MFMA
 
   // S^T = K Q^T for the K tile in stage st
-  auto s_phase = [&](int st) {
-    const unsigned char* kt = smem + st * TILE_B;
+  auto s_phase = [&](const unsigned char* kt) __attribute__((always_inline)) {
 #pragma unroll
     for (int kb = 0; kb < 2; kb++)
 #pragma unroll
       for (int v = 0; v < 16; v++) sacc[kb][v] = 0.f;
     // K fragments are read two k-steps (4 reads) ahead of the MFMAs that use them
     half8_t kf[2][4];
-    auto read_k = [&](int buf, int g) {
+    auto read_k = [&](int buf, int g) __attribute__((always_inline)) {
 #pragma unroll
       for (int u = 0; u < 4; u++)
         kf[buf][u] = *reinterpret_cast<const half8_t*>(kt + (u & 1) * 32 * ROWB + k_rd[2 * g + (u >> 1)]);
@@ -244,7 +287,7 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   };
 
   // online softmax of tile t (per query column, statistics in fp32): sacc -> pf
-  auto softmax_phase = [&](int t) {
+  auto softmax_phase = [&](int t) __attribute__((always_inline)) {
     const int rem = (int)(Skv - (int64_t)t * BKV);  // keys left, this tile included
     const bool ragged = rem < BKV;
     if (PREMUL || ragged) {
@@ -295,13 +338,12 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
 
   // O^T += V^T P^T for the V tile in stage st.
   // k-slot e of lane half `hi` in 16-key step s is key 16*s + 8*(e/4) + 4*hi + (e%4).
-  auto pv_phase = [&](int st) {
-    const unsigned char* vt = smem + (2 + st) * TILE_B;
+  auto pv_phase = [&](const unsigned char* vt) __attribute__((always_inline)) {
     typedef __attribute__((address_space(3))) short4_t lds_s4;
     typedef short short8_t __attribute__((ext_vector_type(8)));
     // V^T fragments of the next 16-key step are read while the current step's MFMAs run
     short4_t vlo[2][DB], vhi[2][DB];
-    auto read_v = [&](int buf, int step) {
+    auto read_v = [&](int buf, int step) __attribute__((always_inline)) {
       const int koff = 16 * step * ROWB;
 #pragma unroll
       for (int db = 0; db < DB; db++) {
@@ -334,32 +376,34 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   // one starts each interval with the softmax of the scores it produced in the
   // previous interval, so one wave's exponentials overlap the other's MFMAs.
   const bool second = wave >= 4;
-  issue_k();   // K(0)
-  stage_k(0);
-  issue_k();   // K(1)
-  issue_v();   // V(0)
+  issue_k(Ks0);  // K(0)
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the tile has landed
   __syncthreads();
 
-  for (int t = 0; t <= n_tiles; t++) {
-    // registers hold K(t+1) and V(t): write them, then start K(t+2) and V(t+1)
-    if (t + 1 < n_tiles) stage_k((t + 1) & 1);
-    if (t < n_tiles) stage_v(t & 1);
-    if (t + 2 < n_tiles) issue_k();
-    if (t + 1 < n_tiles) issue_v();
+  // interval t: K(t) is in k_cur, V(t-1) in v_prev; K(t+1) goes to k_next, V(t) to v_cur
+  auto interval = [&](int t, const unsigned char* k_cur, unsigned char* k_next, const unsigned char* v_prev,
+                      unsigned char* v_cur) __attribute__((always_inline)) {
+    if (t + 1 < n_tiles) issue_k(k_next);
+    if (t < n_tiles) issue_v(v_cur);
     if (!second) {
-      if (t > 0) pv_phase((t - 1) & 1);
+      if (t > 0) pv_phase(v_prev);
       if (t < n_tiles) {
-        s_phase(t & 1);
+        s_phase(k_cur);
         softmax_phase(t);
       }
     } else {
       if (t > 0) {
         softmax_phase(t - 1);
-        pv_phase((t - 1) & 1);
+        pv_phase(v_prev);
       }
-      if (t < n_tiles) s_phase(t & 1);
+      if (t < n_tiles) s_phase(k_cur);
     }
+    __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
+  };
+  for (int t = 0; t <= n_tiles; t += 2) {
+    interval(t, Ks0, Ks1, Vs1, Vs0);
+    if (t + 1 <= n_tiles) interval(t + 1, Ks1, Ks0, Vs0, Vs1);
   }
 
   // ---- normalise and store O ----------------------------------------------
@@ -412,10 +456,18 @@ static dt_status launch(hipStream_t s, SdpaArgs a) {
   int64_t total = (int64_t)a.q_tiles * a.Hq * a.B;
   if (total > 0x7fffffff) return DT_NO_KERNEL;
   a.total_blocks = (int)total;
-  if (a.scale_log2e > 0.f && a.scale_log2e < 1e30f)
-    hipLaunchKernelGGL((sdpa_kernel<DP, false>), dim3((unsigned)total), dim3(512), 0, s, a);
-  else
-    hipLaunchKernelGGL((sdpa_kernel<DP, true>), dim3((unsigned)total), dim3(512), 0, s, a);
+  const bool premul = !(a.scale_log2e > 0.f && a.scale_log2e < 1e30f);
+  // one K and one V segment whose rows lie within 2 GiB of the head's first row: 32-bit offsets
+  const bool oneseg = a.n_kvseg == 1 && a.k[0].ss > 0 && a.v[0].ss > 0 && a.Skv < (1 << 30) &&
+                      (a.Skv + 2 * BKV) * a.k[0].ss * 2 < 0x7fffffffLL && (a.Skv + 2 * BKV) * a.v[0].ss * 2 < 0x7fffffffLL;
+  dim3 grid((unsigned)total), block(512);
+  if (oneseg) {
+    if (premul) hipLaunchKernelGGL((sdpa_kernel<DP, true, true>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((sdpa_kernel<DP, false, true>), grid, block, 0, s, a);
+  } else {
+    if (premul) hipLaunchKernelGGL((sdpa_kernel<DP, true, false>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((sdpa_kernel<DP, false, false>), grid, block, 0, s, a);
+  }
   return launch_status();
 }
 
