@@ -64,4 +64,40 @@ __device__ __forceinline__ float sum32(float v) {
 }
 #endif
 
+// One wave-wide memory -> LDS transfer (global_load_lds_dwordx4): an active
+// lane l's 16 bytes land at LDS byte address lds_base + 16 * l (lds_base
+// wave-uniform).  Written as assembly on purpose: for the builtin the compiler
+// marks a "flat access to both memories" as pending and from then on turns
+// every s_waitcnt it inserts -- LDS counter included -- into a wait for zero
+// until the transfer has landed, which serialises all LDS reads behind it.
+// The caller publishes the data itself: s_waitcnt vmcnt(0) (the transfer
+// counts as a vector memory load; loads return in order, so an outstanding
+// transfer the compiler does not know of can only make one of its own vmcnt
+// waits longer, never too short), then a workgroup barrier, before any wave
+// reads the destination.  M0 is reserved by the compiler, which sets it anew before
+// each of its own uses, so overwriting it here needs no clobber.
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+// source = uniform 64-bit base + 32-bit per-lane byte offset
+__device__ __forceinline__ void load_to_lds_16(const void* gbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds_base), "v"(voff), "s"(gbase)
+      : "memory");
+}
+// source = per-lane 64-bit address
+__device__ __forceinline__ void load_to_lds_16(const void* gptr, uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off"
+      :
+      : "s"(lds_base), "v"(gptr)
+      : "memory");
+}
+
 }  // namespace dt

@@ -96,16 +96,6 @@ __device__ __forceinline__ int pair_chunk(int row, int slot) { return slot ^ ((r
 constexpr int kWaitVm0Lgkm0 = 0x0070;  // s_waitcnt vmcnt(0) lgkmcnt(0)
 constexpr int kWaitLgkm0 = 0xc07f;     // s_waitcnt lgkmcnt(0)
 
-__device__ __forceinline__ uint32_t lds_address(const void* p) {
-  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
-}
-
-// One wave-wide memory -> LDS transfer: lane l's 16 bytes at g land at LDS
-// address lds + 16 * l (lds wave-uniform).
-__device__ __forceinline__ void load_to_lds_16(const void* g, half_t* lds) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                   (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
-}
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
   return (uint32_t)half_to_bits((half_t)a) | ((uint32_t)half_to_bits((half_t)b) << 16);
@@ -299,9 +289,9 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
 #endif
     const int64_t kb = (int64_t)q * (4 * BK);  // byte offset of the pair inside a row
     if (i < AP) {
-      load_to_lds_16(xbase + kb + a_off[i], xs + (wave_u * AP + i) * 512);
+      load_to_lds_16(xbase + kb, a_off[i], lds_address(xs) + (uint32_t)((wave_u * AP + i) * 1024));
     } else if constexpr (MODE == kPlainF16) {
-      load_to_lds_16(wbase + kb + bf_off[i - AP], wp + (wave_u * BP + i - AP) * 512);
+      load_to_lds_16(wbase + kb, bf_off[i - AP], lds_address(wp) + (uint32_t)((wave_u * BP + i - AP) * 1024));
     }
   };
   auto issue_pair = [&](half_t* xs, half_t* wp, int q) {

@@ -29,12 +29,6 @@ typedef short short4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// One wave-wide memory -> LDS transfer: an active lane l's 16 bytes at g land
-// at LDS address lds + 16 * l (lds wave-uniform).
-__device__ __forceinline__ void load_to_lds_16(const void* g, unsigned char* lds) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                   (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
-}
 // LDS layouts (measured bank-conflict free on this part: 64 banks, 16 lanes of
 // a 16-byte access or 32 lanes of an 8-byte access per clock).
 // K tile: [64 keys][DP] halfs; 16-byte chunk c of key row r is stored at a
@@ -195,10 +189,10 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
       if constexpr (ONESEG) {
-        if (ld_row[i] < rows_left && k_ch[i] * 8 < D) load_to_lds_16(k_base + k_off[i], dst + (wave_u * LOADS + i) * 1024);
+        if (ld_row[i] < rows_left && k_ch[i] * 8 < D) load_to_lds_16(k_base, k_off[i], lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
         k_off[i] += k_step;
       } else {
-        if (kp[i].row < Skv && k_ch[i] * 8 < D) load_to_lds_16(kp[i].p, dst + (wave_u * LOADS + i) * 1024);
+        if (kp[i].row < Skv && k_ch[i] * 8 < D) load_to_lds_16(kp[i].p, lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
         advance(a.k, k_ch[i], kp[i]);
       }
     }
@@ -208,10 +202,10 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
       if constexpr (ONESEG) {
-        if (ld_row[i] < rows_left_v && v_ch[i] * 8 < D) load_to_lds_16(v_base + v_off[i], dst + (wave_u * LOADS + i) * 1024);
+        if (ld_row[i] < rows_left_v && v_ch[i] * 8 < D) load_to_lds_16(v_base, v_off[i], lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
         v_off[i] += v_step;
       } else {
-        if (vp[i].row < Skv && v_ch[i] * 8 < D) load_to_lds_16(vp[i].p, dst + (wave_u * LOADS + i) * 1024);
+        if (vp[i].row < Skv && v_ch[i] * 8 < D) load_to_lds_16(vp[i].p, lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
         advance(a.v, v_ch[i], vp[i]);
       }
     }
@@ -288,6 +282,16 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
 
   // online softmax of tile t (per query column, statistics in fp32): sacc -> pf
   auto softmax_phase = [&](int t) __attribute__((always_inline)) {
+#ifdef DT_EXP_NOSOFTMAX
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+      for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) pf[kb][tt][e] = (half_t)(sacc[kb][8 * tt + e] * 1e-3f);
+    l_run = 1.f;
+    return;
+#endif
     const int rem = (int)(Skv - (int64_t)t * BKV);  // keys left, this tile included
     const bool ragged = rem < BKV;
     if (PREMUL || ragged) {
@@ -329,7 +333,13 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       for (int tt = 0; tt < 2; tt++)
 #pragma unroll
         for (int e = 0; e < 8; e++) {
+#if defined(DT_EXP_NOEXP)
+          const float p = __builtin_fmaf(sacc[kb][8 * tt + e], c, -mc) * 1e-3f;
+#elif defined(DT_EXP_EXPONLY)
+          const float p = fast_exp2(sacc[kb][8 * tt + e]);
+#else
           const float p = fast_exp2(__builtin_fmaf(sacc[kb][8 * tt + e], c, -mc));
+#endif
           psum += p;
           pf[kb][tt][e] = (half_t)p;
         }
@@ -383,9 +393,15 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   // interval t: K(t) is in k_cur, V(t-1) in v_prev; K(t+1) goes to k_next, V(t) to v_cur
   auto interval = [&](int t, const unsigned char* k_cur, unsigned char* k_next, const unsigned char* v_prev,
                       unsigned char* v_cur) __attribute__((always_inline)) {
+#ifndef DT_EXP_NODMA
     if (t + 1 < n_tiles) issue_k(k_next);
     if (t < n_tiles) issue_v(v_cur);
+#endif
+#ifdef DT_EXP_NOSKEW
+    if (true) {
+#else
     if (!second) {
+#endif
       if (t > 0) pv_phase(v_prev);
       if (t < n_tiles) {
         s_phase(k_cur);
