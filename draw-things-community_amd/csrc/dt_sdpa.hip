@@ -125,40 +125,11 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     k_ch[i] = k_chunk_swz<DP>(row, pc);  // the swizzles are involutions
     v_ch[i] = v_unit_swz<DP>(row, pc >> 2) * 4 + (pc & 3);
   }
-  struct RowPtr {
-    const uint16_t* p;  // chunk address of the current row
-    int64_t row;        // joint row index
-    int64_t end;        // first joint row past the current segment
-    int64_t step;       // elements per 64 rows inside the current segment
-  };
-  auto locate = [&](const SdpaSeg* segs, int64_t kj, int ch, RowPtr& r) __attribute__((always_inline)) {
-    int sg = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxSeg; i++)
-      if (i < a.n_kvseg && kj >= segs[i].start) sg = i;
-    r.p = segs[sg].ptr + b * segs[sg].sb + (kj - segs[sg].start) * segs[sg].ss + hk * segs[sg].sh + ch * 8;
-    r.row = kj;
-    r.end = (sg + 1 < a.n_kvseg) ? segs[sg + 1].start : Skv;
-    r.step = segs[sg].ss * BKV;
-  };
-  const bool one_seg = a.n_kvseg == 1;  // uniform
-  auto advance = [&](const SdpaSeg* segs, int ch, RowPtr& r) __attribute__((always_inline)) {
-    const int64_t kj = r.row + BKV;
-    if (one_seg) {  // uniform: rows past the end are never dereferenced
-      r.row = kj;
-      r.p += r.step;
-    } else if (kj < r.end) {
-      r.row = kj;
-      r.p += r.step;
-    } else if (kj < Skv) {
-      locate(segs, kj, ch, r);
-    } else {
-      r.row = kj;
-    }
-  };
-  RowPtr kp[ONESEG ? 1 : LOADS], vp[ONESEG ? 1 : LOADS];
   // ONESEG: K and V are one run of rows each and small enough for 32-bit byte
   // offsets from a uniform base; a tile step adds a uniform stride.
+  // Otherwise the segment of a tile is looked up once per tile (uniformly): a
+  // tile that lies inside one segment is fetched from that segment's base with
+  // per-lane 32-bit offsets, a tile that straddles segments row by row.
   uint32_t k_off[LOADS], v_off[LOADS];
   const char* k_base = nullptr;
   const char* v_base = nullptr;
@@ -175,41 +146,89 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       k_off[i] = (uint32_t)((ld_row[i] * a.k[0].ss + k_ch[i] * 8) * 2);
       v_off[i] = (uint32_t)((ld_row[i] * a.v[0].ss + v_ch[i] * 8) * 2);
     }
-  } else {
-#pragma unroll
-    for (int i = 0; i < LOADS; i++) {
-      locate(a.k, ld_row[i] < Skv ? ld_row[i] : 0, k_ch[i], kp[i]);
-      kp[i].row = ld_row[i];
-      locate(a.v, ld_row[i] < Skv ? ld_row[i] : 0, v_ch[i], vp[i]);
-      vp[i].row = ld_row[i];
-    }
   }
-  // starts the transfer of the K (or V) tile the pointers stand on, then moves them to the next tile
-  auto issue_k = [&](unsigned char* dst) __attribute__((always_inline)) {
+  // General case: a uniform cursor holds the segment the next tile starts in --
+  // address of the tile's first row, row stride, last row of the segment --
+  // and is re-read from the argument block only when a tile starts past that
+  // segment's end.  Tiles inside the segment are fetched with per-lane 32-bit
+  // offsets from the cursor; a tile that straddles segments goes row by row.
+  struct SegCursor {
+    const char* base;  // first row of the next tile (this batch and head)
+    int64_t ss;        // row stride, elements
+    int64_t end;       // first joint row past the segment
+    int64_t row0;      // first joint row of the next tile
+  };
+  SegCursor kcur{nullptr, 0, 0, 0}, vcur{nullptr, 0, 0, 0};
+  auto seek = [&](const SdpaSeg* segs, SegCursor& c, uint32_t (&off)[LOADS], const int (&chs)[LOADS])
+                  __attribute__((always_inline)) {
+    int sg = 0;
 #pragma unroll
-    for (int i = 0; i < LOADS; i++) {
-      if constexpr (ONESEG) {
-        if (ld_row[i] < rows_left && k_ch[i] * 8 < D) load_to_lds_16(k_base, k_off[i], lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
-        k_off[i] += k_step;
+    for (int i = 1; i < kMaxSeg; i++)
+      if (i < a.n_kvseg && c.row0 >= segs[i].start) sg = i;
+    c.ss = segs[sg].ss;
+    c.end = (sg + 1 < a.n_kvseg) ? segs[sg + 1].start : Skv;
+    c.base = reinterpret_cast<const char*>(segs[sg].ptr + b * segs[sg].sb + hk * segs[sg].sh +
+                                           (c.row0 - segs[sg].start) * c.ss);
+#pragma unroll
+    for (int i = 0; i < LOADS; i++) off[i] = (uint32_t)((ld_row[i] * c.ss + chs[i] * 8) * 2);
+  };
+  auto issue_general = [&](const SdpaSeg* segs, SegCursor& c, uint32_t (&off)[LOADS], const int (&chs)[LOADS],
+                           unsigned char* dst) __attribute__((always_inline)) {
+    if (c.row0 < Skv) {
+      if (c.row0 >= c.end) seek(segs, c, off, chs);  // uniform
+      const int64_t last = c.row0 + BKV < Skv ? c.row0 + BKV : Skv;
+      if (last <= c.end && c.ss > 0 && c.ss < (1 << 24)) {
+        const int n_rows = (int)(last - c.row0);
+        const void* base = c.base;
+#pragma unroll
+        for (int i = 0; i < LOADS; i++)
+          if (ld_row[i] < n_rows && chs[i] * 8 < D)
+            load_to_lds_16(base, off[i], lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
       } else {
-        if (kp[i].row < Skv && k_ch[i] * 8 < D) load_to_lds_16(kp[i].p, lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
-        advance(a.k, k_ch[i], kp[i]);
+#pragma unroll
+        for (int i = 0; i < LOADS; i++) {
+          const int64_t kj = c.row0 + ld_row[i];
+          if (kj < Skv && chs[i] * 8 < D) {
+            int sl = 0;
+#pragma unroll
+            for (int u = 1; u < kMaxSeg; u++)
+              if (u < a.n_kvseg && kj >= segs[u].start) sl = u;
+            const uint16_t* src =
+                segs[sl].ptr + b * segs[sl].sb + (kj - segs[sl].start) * segs[sl].ss + hk * segs[sl].sh + chs[i] * 8;
+            load_to_lds_16(src, lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
+          }
+        }
       }
     }
-    rows_left -= BKV;
+    c.base += c.ss * (BKV * 2);
+    c.row0 += BKV;
+  };
+  // starts the transfer of the next K (or V) tile and moves on by one tile
+  auto issue_k = [&](unsigned char* dst) __attribute__((always_inline)) {
+    if constexpr (ONESEG) {
+#pragma unroll
+      for (int i = 0; i < LOADS; i++) {
+        if (ld_row[i] < rows_left && k_ch[i] * 8 < D)
+          load_to_lds_16(k_base, k_off[i], lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
+        k_off[i] += k_step;
+      }
+      rows_left -= BKV;
+    } else {
+      issue_general(a.k, kcur, k_off, k_ch, dst);
+    }
   };
   auto issue_v = [&](unsigned char* dst) __attribute__((always_inline)) {
+    if constexpr (ONESEG) {
 #pragma unroll
-    for (int i = 0; i < LOADS; i++) {
-      if constexpr (ONESEG) {
-        if (ld_row[i] < rows_left_v && v_ch[i] * 8 < D) load_to_lds_16(v_base, v_off[i], lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
+      for (int i = 0; i < LOADS; i++) {
+        if (ld_row[i] < rows_left_v && v_ch[i] * 8 < D)
+          load_to_lds_16(v_base, v_off[i], lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
         v_off[i] += v_step;
-      } else {
-        if (vp[i].row < Skv && v_ch[i] * 8 < D) load_to_lds_16(vp[i].p, lds_address(dst) + (uint32_t)((wave_u * LOADS + i) * 1024));
-        advance(a.v, v_ch[i], vp[i]);
       }
+      rows_left_v -= BKV;
+    } else {
+      issue_general(a.v, vcur, v_off, v_ch, dst);
     }
-    rows_left_v -= BKV;
   };
   // slots that no transfer will ever write must not hold NaN patterns
   if (D < DP || Skv % BKV != 0) {

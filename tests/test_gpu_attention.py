@@ -184,6 +184,26 @@ def test_sdpa_segments_equal_concat_and_strided_views(dthip, oracle, torch_cuda)
     assert np.array_equal(cat.cpu().numpy().view(np.uint16), got.view(np.uint16))
 
 
+@pytest.mark.parametrize("lens,D", [((5, 130, 1, 64), 64), ((64, 64, 200), 128), ((3, 2, 1, 70), 40)])
+def test_sdpa_many_segments(dthip, oracle, torch_cuda, lens, D):
+    """Up to four K/V segments, some shorter than a 64-key tile (several segment boundaries inside one tile) and some
+    ending on a tile boundary: bit-identical to the concatenated call, and equal to the oracle."""
+    torch = torch_cuda
+    rng = np.random.default_rng(sum(lens) + D)
+    B, Hq, Hk = 2, 4, 2
+    ks = [f16(rng.standard_normal((B, n, Hk, D))) for n in lens]
+    vs = [f16(rng.standard_normal((B, n, Hk, D))) for n in lens]
+    q = f16(rng.standard_normal((B, 90, Hq, D)))
+    scale = 1 / np.sqrt(D)
+    print("sdpa many segments", lens, D, flush=True)
+    got = dthip.sdpa_segments([to_dev(torch, q)], [to_dev(torch, t) for t in ks], [to_dev(torch, t) for t in vs], scale)
+    k, v = np.concatenate(ks, axis=1), np.concatenate(vs, axis=1)
+    cat = dthip.ScaledDotProductAttention(scale=scale)(to_dev(torch, q), to_dev(torch, k), to_dev(torch, v))
+    assert torch.equal(got, cat)
+    mx, rr = oracle.err_stats(got.cpu().numpy(), oracle.C.sdpa(q, k, v, scale))
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
 def test_sdpa_fused_norm_rope_joint(dthip, oracle, torch_cuda):
     """The Flux joint block's attention input stage fused into the call: per-segment per-head RMSNorm
     (c_norm_* / x_norm_*), RoPE over the joint order, then attention."""
