@@ -31,6 +31,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="launch the step's kernels one by one instead of as a HIP graph")
     ap.add_argument("--kernel-iters", type=int, default=20, help="launches per kernel for the per-kernel timings")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
@@ -136,12 +137,42 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    # The step is three dependent launches; replayed as a HIP graph they go out without host gaps.  The graph is
+    # used only if its replays, with eager work in between, reproduce the eager outputs bit for bit.
+    run_step, launch_mode = step, "eager"
+    if not args.no_graph:
+        try:
+            step()
+            torch.cuda.synchronize()
+            want = (out_x.clone(), out_c.clone(), att.clone())
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            ok = True
+            for _ in range(3):
+                out_x.zero_(); out_c.zero_(); att.zero_()
+                graph.replay()
+                torch.cuda.synchronize()
+                ok = ok and all(torch.equal(a_, b_) for a_, b_ in zip((out_x, out_c, att), want))
+                step()  # eager work between replays
+                torch.cuda.synchronize()
+            if ok:
+                run_step, launch_mode = graph.replay, "hip graph (3 kernels)"
+        except Exception as e:  # capture not possible: stay eager
+            print(f"graph capture failed, running eagerly: {e}", file=sys.stderr)
+            torch.cuda.synchronize()
+
     for _ in range(args.warmup):
-        step()
+        run_step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        run_step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / max(args.steps, 1)
     value = flop_block / (ms_per_step * 1e-3) / 1e12
@@ -230,22 +261,28 @@ def main():
         t0 = time.perf_counter()
         xs_c = rng.standard_normal((T, C)).astype(np.float16)
         xs_x = rng.standard_normal((HW, C)).astype(np.float16)
-        t0 = time.perf_counter()
-        for name in ("c_q", "c_k", "c_v", "c_o"):
-            oracle.C.dense_qx(xs_c, packed_host[name], qbits, nib, C, None)
-        for name in ("x_q", "x_k", "x_v", "x_o"):
-            oracle.C.dense_qx(xs_x, packed_host[name], qbits, nib, C, None)
-        t_dense = time.perf_counter() - t0
         qs = rng.standard_normal((1, S, H, D)).astype(np.float16)
         ks = rng.standard_normal((1, S, H, D)).astype(np.float16)
         vs = rng.standard_normal((1, S, H, D)).astype(np.float16)
-        t0 = time.perf_counter()
-        oracle.C.sdpa(qs, ks, vs, scale)
-        t_sdpa = time.perf_counter() - t0
+        t_dense = t_sdpa = 0.0
+        passes = 0
+        while passes < 8 and t_dense + t_sdpa < 12.0:  # whole blocks until ~12 s of CPU work
+            t0 = time.perf_counter()
+            for name in ("c_q", "c_k", "c_v", "c_o"):
+                oracle.C.dense_qx(xs_c, packed_host[name], qbits, nib, C, None)
+            for name in ("x_q", "x_k", "x_v", "x_o"):
+                oracle.C.dense_qx(xs_x, packed_host[name], qbits, nib, C, None)
+            t1 = time.perf_counter()
+            oracle.C.sdpa(qs, ks, vs, scale)
+            t_sdpa += time.perf_counter() - t1
+            t_dense += t1 - t0
+            passes += 1
+        t_dense /= passes
+        t_sdpa /= passes
         t_block = t_dense + t_sdpa
         cpu = {
             "value": round(flop_block / t_block / 1e12, 5), "unit": "TFLOP/s", "cores": int(ncores), "kind": "port",
-            "sample": f"oracle (C, OpenMP, {ncores} threads), the whole block at full size, one pass: 8 q6p Dense "
+            "sample": f"oracle (C, OpenMP, {ncores} threads), the whole block at full size, mean of {passes} passes: 8 q6p Dense "
                       f"3072->3072 (512 / 4096 rows, depalettize included, {t_dense:.2f} s) + attention 24 heads x 4608 x 4608 "
                       f"({t_sdpa:.2f} s); RMSNorm/RoPE not included",
             "ms_per_block": round(t_block * 1e3, 1),
@@ -256,7 +293,7 @@ def main():
         "metric": "SDPA + palettized-GEMM TFLOP/s (% fp16 peak); ms/block, Flux 4608 tok q6p",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
+        "dtype": "f16", "data": "synthetic", "launch": launch_mode,
         "config": {"workload": "Flux.1-dev joint attention block hot path: 512 text + 4096 image tokens, 24x128 heads, "
                                "q6p (nib 4096) weights; 6 QKV Dense (QK RMSNorm/RoPE fused in the epilogue) + SDPA + 2 out-proj Dense",
                    "flop_per_block": flop_block, "frac_f16_peak": round(value / PEAK_F16_TFLOPS, 4)},

@@ -433,7 +433,9 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       }
       if (t < n_tiles) s_phase(k_cur);
     }
+#ifndef DT_EXP_NOWAIT
     __builtin_amdgcn_s_waitcnt(0x0f70);
+#endif
     __syncthreads();
   };
   for (int t = 0; t <= n_tiles; t += 2) {
