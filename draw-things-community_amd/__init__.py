@@ -33,6 +33,7 @@ ABI_SYMBOLS = (
     "dt_dense_qx_f16",
     "dt_dense_qx_heads_f16",
     "dt_dense_qx_grouped_f16",
+    "dt_dense_qx_post_f16",
     "dt_qk_norm_rope_f16",
     "dt_sdpa_f16",
     "dt_sdpa_workspace_bytes",
@@ -57,6 +58,11 @@ class _View4(ctypes.Structure):
 class _HeadEpilogue(ctypes.Structure):
     _fields_ = [("gamma", ctypes.c_void_p), ("rot", ctypes.c_void_p), ("rot_pos0", ctypes.c_int64),
                 ("eps", ctypes.c_float), ("head_dim", ctypes.c_int32)]
+
+
+class _DensePost(ctypes.Structure):
+    _fields_ = [("activation", ctypes.c_int32), ("gate", ctypes.c_void_p), ("residual", ctypes.c_void_p),
+                ("ld_residual", ctypes.c_int64)]
 
 
 class _DenseGroup(ctypes.Structure):
@@ -110,6 +116,10 @@ def lib():
                                             ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(i64),
                                             ctypes.POINTER(_HeadEpilogue), ctypes.c_uint32]
         L.dt_qk_norm_rope_f16.restype = i32
+        L.dt_dense_qx_post_f16.restype = i32
+        L.dt_dense_qx_post_f16.argtypes = [vp, i64, i64, vp, i64, ctypes.POINTER(_QxWeight), i32,
+                                           ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(i64),
+                                           ctypes.POINTER(_DensePost), ctypes.c_uint32]
         L.dt_dense_qx_grouped_f16.restype = i32
         L.dt_dense_qx_grouped_f16.argtypes = [vp, i32, ctypes.POINTER(_DenseGroup), ctypes.c_uint32]
         L.dt_qk_norm_rope_f16.argtypes = [vp, _View4, i32, i64, i32, i32, vp, f32, i32, vp, i64, f32]
@@ -336,6 +346,53 @@ def dense_multi(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object
         st = lib().dt_dense_qx_heads_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, E, flags)
         _check("dt_dense_qx_heads_f16", st)
     return _shape_outs(x, M, outs)
+
+
+ACT_NONE, ACT_GELU_TANH, ACT_SWISH = 0, 1, 2
+
+
+class DensePost:
+    """Elementwise tail of one projection: activation (ACT_*), per-feature fp16 gate [N], fp32 residual [M, N] that the
+    result is accumulated into (`x + (y .* gate).to(of: x)`, Models/Flux1.swift:250).  With `residual` given and
+    `keep_output=False` the fp16 result itself is not written."""
+
+    def __init__(self, activation: int = ACT_NONE, gate=None, residual=None, keep_output: bool = True):
+        self.activation, self.gate, self.residual, self.keep_output = activation, gate, residual, keep_output
+
+
+def dense_post(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]], posts: Sequence[Optional[DensePost]],
+               outs=None, flags: int = 0, stream=None):
+    """Dense ops sharing `x`, each followed by its DensePost tail inside the GEMM epilogue (the feed-forward's
+    linear1 -> GELU and the gated residual additions of a transformer block).  Returns the fp16 outputs (None where
+    a projection only accumulates into its residual)."""
+    torch = _torch()
+    x2, M, K, n, W, B, Y, LDY, _, outs = _marshal_dense(x, weights, biases, outs, None)
+    P = (_DensePost * n)()
+    for i, p in enumerate(posts):
+        if p is None:
+            P[i] = _DensePost(ACT_NONE, None, None, 0)
+            continue
+        N = weights[i].shape[0]
+        if p.gate is not None and (_f16_cuda(p.gate, "gate").numel() != N or not p.gate.is_contiguous()):
+            raise ValueError("gate must hold one value per output feature")
+        rp, ldr = None, 0
+        if p.residual is not None:
+            r = p.residual
+            if not (isinstance(r, torch.Tensor) and r.is_cuda and r.dtype == torch.float32):
+                raise TypeError("residual must be a float32 CUDA tensor")
+            r2 = r.reshape(-1, N) if r.dim() != 2 else r
+            if r2.shape != (M, N) or r2.stride(1) != 1 or r2.data_ptr() != r.data_ptr():
+                raise ValueError("residual must be an [M, N] view with contiguous rows")
+            rp, ldr = r2.data_ptr(), r2.stride(0)
+            if not p.keep_output:
+                Y[i] = None
+                outs[i] = None
+        P[i] = _DensePost(p.activation, None if p.gate is None else p.gate.data_ptr(), rp, ldr)
+    st = lib().dt_dense_qx_post_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, P, flags)
+    _check("dt_dense_qx_post_f16", st)
+    lead = tuple(x.shape[:-1])
+    return [None if o is None else (o.reshape(lead + (o.shape[-1],)) if o.shape[0] == M and o.is_contiguous() else o)
+            for o in outs]
 
 
 def dense_grouped(problems: Sequence[dict], flags: int = 0, stream=None):

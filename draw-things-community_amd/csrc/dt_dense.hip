@@ -43,7 +43,30 @@ struct DenseWeight {
   const uint16_t* rot;
   int64_t rot_pos0;
   float eps;
+  // optional elementwise tail: activation, per-feature gate, accumulation into an fp32 residual stream
+  int32_t act;          // DT_ACT_*
+  const uint16_t* gate;  // [n] or null
+  float* res;            // [m, n] fp32 with row stride ld_res, updated in place; null = none
+  int64_t ld_res;
 };
+
+// The elementwise tail on one value that has already been rounded to fp16, with
+// the rounding the op-by-op graph applies: after the activation and after the gate.
+__device__ __forceinline__ float act_gelu_tanh(float x) {
+  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  const float e = __builtin_amdgcn_exp2f(u * 2.885390081777927f);  // exp(2u)
+  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);   // tanh(u)
+  return 0.5f * x * (1.0f + t);
+}
+__device__ __forceinline__ float act_swish(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+__device__ __forceinline__ float post_value(float v, int act, bool has_gate, float gate) {
+  if (act == DT_ACT_GELU_TANH) v = (float)(half_t)act_gelu_tanh(v);
+  else if (act == DT_ACT_SWISH) v = (float)(half_t)act_swish(v);
+  if (has_gate) v = (float)(half_t)(v * gate);
+  return v;
+}
 
 // One X with the weights applied to it; a launch runs up to kMaxGroups of them
 // (same K and weight format), their tiles numbered one group after the other.
@@ -110,7 +133,7 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 // eight run MFMAs on a (BN/2) x (BM/4) slice.  The accumulators are held
 // transposed (rows = output features n, columns = tokens m) so that each lane
 // ends up with runs of consecutive n for one token: 16-byte stores.
-template <int Q, int BM, int BN, int MODE>
+template <int Q, int BM, int BN, int MODE, bool POST>
 __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   constexpr int WN = BN / 2, WM = BM / 4;   // per-wave slice: WN features x WM tokens
   constexpr int TN = WN / 32, TM = WM / 32;
@@ -563,6 +586,75 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     iteration(t + 1, 1, XsA, WpA, XsB, WpB);
   }
 
+  // ---- epilogue with an elementwise tail (activation, gate, fp32 residual) -------
+  // Straight from the accumulators: lane holds token column (lane & 31) and runs
+  // of 4 consecutive features 8 * g + 4 * (lane / 32) + (0..3) per block.
+  if constexpr (POST) {
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      const int gm = m0 + wm * WM + j * 32 + l32;
+      const int64_t gmc = gm < g.m ? gm : 0;
+      uint16_t* yrow = w.y ? w.y + gmc * w.ldy : nullptr;
+      float* rrow = w.res ? w.res + gmc * w.ld_res : nullptr;
+      const bool vec = (!w.gate || (reinterpret_cast<uintptr_t>(w.gate) & 7) == 0) &&
+                       (!w.bias || (reinterpret_cast<uintptr_t>(w.bias) & 7) == 0) &&
+                       (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0)) &&
+                       (!w.y || (((w.ldy & 3) == 0) && (reinterpret_cast<uintptr_t>(w.y) & 7) == 0));
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int gq = 0; gq < 4; gq++) {
+          const int nn = n0 + wn * WN + i * 32 + 8 * gq + 4 * hi;
+          float bq[4] = {0.f, 0.f, 0.f, 0.f}, gt[4] = {1.f, 1.f, 1.f, 1.f}, rr[4] = {0.f, 0.f, 0.f, 0.f}, pv[4];
+          const bool full = vec && nn + 3 < w.n;
+          if (gm < g.m) {
+            if (full) {
+              if (w.bias) {
+                const uint2_t t2 = *reinterpret_cast<const uint2_t*>(w.bias + nn);
+                bq[0] = (float)bits_to_half((uint16_t)t2[0]); bq[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
+                bq[2] = (float)bits_to_half((uint16_t)t2[1]); bq[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
+              }
+              if (w.gate) {
+                const uint2_t t2 = *reinterpret_cast<const uint2_t*>(w.gate + nn);
+                gt[0] = (float)bits_to_half((uint16_t)t2[0]); gt[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
+                gt[2] = (float)bits_to_half((uint16_t)t2[1]); gt[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
+              }
+              if (rrow) {
+                const float4_t t4 = *reinterpret_cast<const float4_t*>(rrow + nn);
+                rr[0] = t4[0]; rr[1] = t4[1]; rr[2] = t4[2]; rr[3] = t4[3];
+              }
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                if (nn + e < w.n) {
+                  if (w.bias) bq[e] = (float)bits_to_half(w.bias[nn + e]);
+                  if (w.gate) gt[e] = (float)bits_to_half(w.gate[nn + e]);
+                  if (rrow) rr[e] = rrow[nn + e];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const float v0 = (float)(half_t)(acc[i][j][4 * gq + e] + bq[e]);
+              pv[e] = post_value(v0, w.act, w.gate != nullptr, gt[e]);
+              rr[e] += pv[e];
+            }
+            if (full) {
+              if (rrow) *reinterpret_cast<float4_t*>(rrow + nn) = float4_t{rr[0], rr[1], rr[2], rr[3]};
+              if (yrow) *reinterpret_cast<uint2_t*>(yrow + nn) = uint2_t{pack_h2(pv[0], pv[1]), pack_h2(pv[2], pv[3])};
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                if (nn + e < w.n) {
+                  if (rrow) rrow[nn + e] = rr[e];
+                  if (yrow) yrow[nn + e] = half_to_bits((half_t)pv[e]);
+                }
+            }
+          }
+        }
+    }
+    return;
+  }
+
   // ---- fused epilogue: per-head RMSNorm and RoPE on the way out ---------------
   // A wave's 128 features are exactly one head, and every lane pair (l, l ^ 32)
   // holds all 128 of them for its token, adjacent (re, im) pairs in one lane:
@@ -720,7 +812,9 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
 __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* __restrict__ x, int64_t ldx, int64_t m,
                                                              int64_t n, int64_t k, const uint8_t* __restrict__ wdata,
                                                              int qbits, int nib, const uint16_t* __restrict__ bias,
-                                                             uint16_t* __restrict__ y, int64_t ldy) {
+                                                             uint16_t* __restrict__ y, int64_t ldy, int act,
+                                                             const uint16_t* __restrict__ gate, float* __restrict__ res,
+                                                             int64_t ld_res) {
   int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (o >= m * n) return;
   int64_t mi = o / n, ni = o - mi * n;
@@ -741,41 +835,52 @@ __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* _
     }
   }
   if (bias) acc += (float)bits_to_half(bias[ni]);
-  y[mi * ldy + ni] = half_to_bits((half_t)acc);
+  float v = (float)(half_t)acc;
+  v = post_value(v, act, gate != nullptr, gate ? (float)bits_to_half(gate[ni]) : 1.0f);
+  if (res) res[mi * ld_res + ni] += v;
+  if (y) y[mi * ldy + ni] = half_to_bits((half_t)v);
 }
 
-template <int Q, int BM, int BN>
+template <int Q, int BM, int BN, bool POST>
 static dt_status launch_tiled(hipStream_t s, const DenseArgs& a, int mode) {
   dim3 grid((unsigned)a.total_tiles), block(512);
   switch (mode) {
-    case kPalShared: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalShared>), grid, block, 0, s, a); break;
+    case kPalShared: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalShared, POST>), grid, block, 0, s, a); break;
     case kPalRow:
       if constexpr ((BN << (Q + 1)) <= kPalLdsBytes) {
-        hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalRow>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalRow, POST>), grid, block, 0, s, a);
         break;
       } else {
         return DT_NO_KERNEL;  // choose_pal_mode never picks per-row palettes that do not fit
       }
-    default: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalGlobal>), grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalGlobal, POST>), grid, block, 0, s, a); break;
   }
   return launch_status();
 }
 
-template <int BM, int BN>
-static dt_status launch_tiled_q(hipStream_t s, const DenseArgs& a, int qbits, int mode) {
+template <int BM, int BN, bool POST>
+static dt_status launch_tiled_qp(hipStream_t s, const DenseArgs& a, int qbits, int mode) {
   switch (qbits) {
-    case 4: return launch_tiled<4, BM, BN>(s, a, mode);
-    case 5: return launch_tiled<5, BM, BN>(s, a, mode);
-    case 6: return launch_tiled<6, BM, BN>(s, a, mode);
-    case 7: return launch_tiled<7, BM, BN>(s, a, mode);
-    case 8: return launch_tiled<8, BM, BN>(s, a, mode);
+    case 4: return launch_tiled<4, BM, BN, POST>(s, a, mode);
+    case 5: return launch_tiled<5, BM, BN, POST>(s, a, mode);
+    case 6: return launch_tiled<6, BM, BN, POST>(s, a, mode);
+    case 7: return launch_tiled<7, BM, BN, POST>(s, a, mode);
+    case 8: return launch_tiled<8, BM, BN, POST>(s, a, mode);
     case 16: {
       dim3 grid((unsigned)a.total_tiles), block(512);
-      hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16>), grid, block, 0, s, a);
+      hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, POST>), grid, block, 0, s, a);
       return launch_status();
     }
   }
   return DT_INVALID;
+}
+
+// the kernel with the elementwise tail only when some weight of the launch asks for one
+template <int BM, int BN>
+static dt_status launch_tiled_q(hipStream_t s, const DenseArgs& a, int qbits, int mode) {
+  bool post = false;
+  for (int i = 0; i < kMaxWeights; i++) post = post || a.w[i].act != DT_ACT_NONE || a.w[i].gate || a.w[i].res;
+  return post ? launch_tiled_qp<BM, BN, true>(s, a, qbits, mode) : launch_tiled_qp<BM, BN, false>(s, a, qbits, mode);
 }
 
 // Palette placement for a BN-row tile (see PalMode).
@@ -803,6 +908,7 @@ struct HostGroup {
   uint16_t* const* Y;
   const int64_t* ldy;
   const dt_head_epilogue* epi;
+  const dt_dense_post* post;
 
   bool wants_epi(int wi) const { return epi && (epi[wi].gamma || epi[wi].rot); }
   // fused head epilogue: in the tiled kernel for 128-wide heads that start on a 16-byte aligned,
@@ -835,13 +941,22 @@ static dt_status validate_group(const HostGroup& h) {
     }
   }
   if (h.M < 0 || h.K <= 0 || h.n_weights <= 0 || !h.W || !h.Y || !h.ldy) return DT_INVALID;
+  if (h.post && h.epi) return DT_INVALID;
+  if (h.post)
+    for (int i = 0; i < h.n_weights; i++) {
+      const dt_dense_post& p = h.post[i];
+      if (p.activation < DT_ACT_NONE || p.activation > DT_ACT_SWISH) return DT_INVALID;
+      if (p.residual && ((reinterpret_cast<uintptr_t>(p.residual) & 3) || (h.W && h.K > 0 && p.ld_residual < h.W[i].count / h.K)))
+        return DT_INVALID;
+    }
   if (h.M > 0x7fffffff || h.K > 0x7fffffff) return DT_INVALID;
   for (int i = 0; i < h.n_weights; i++) {
     const dt_qx_weight& w = h.W[i];
     if (!w.data || w.count < 0 || w.count % h.K != 0) return DT_INVALID;
     if (w.qbits != 16 && (w.qbits < 4 || w.qbits > 8 || w.nib <= 0)) return DT_INVALID;
     if (w.count / h.K > 0x7fffffff) return DT_INVALID;
-    if (h.M > 0 && (!h.Y[i] || h.ldy[i] < w.count / h.K)) return DT_INVALID;
+    const bool to_residual_only = h.post && h.post[i].residual && !h.Y[i];
+    if (h.M > 0 && !to_residual_only && (!h.Y[i] || h.ldy[i] < w.count / h.K)) return DT_INVALID;
   }
   if (h.M > 0 && (!h.X || h.ldx < h.K)) return DT_INVALID;
   return DT_OK;
@@ -881,6 +996,10 @@ static int add_weight(DenseArgs& a, int slot, const HostGroup& h, int wi, int ti
   d.rot = fuse ? h.epi[wi].rot : nullptr;
   d.rot_pos0 = fuse ? h.epi[wi].rot_pos0 : 0;
   d.eps = fuse ? h.epi[wi].eps : 0.f;
+  d.act = h.post ? h.post[wi].activation : DT_ACT_NONE;
+  d.gate = h.post ? h.post[wi].gate : nullptr;
+  d.res = h.post ? h.post[wi].residual : nullptr;
+  d.ld_res = h.post ? h.post[wi].ld_residual : 0;
   return (int)((n_rows + BN - 1) / BN);
 }
 
@@ -909,7 +1028,9 @@ static dt_status run_group(hipStream_t s, const HostGroup& h) {
         if ((outs + 255) / 256 > 0x7fffffff) return DT_NO_KERNEL;
         hipLaunchKernelGGL(dense_qx_generic_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, s, h.X, h.ldx,
                            M, n_rows0, K, static_cast<const uint8_t*>(w0.data), w0.qbits, w0.nib,
-                           h.bias ? h.bias[i] : nullptr, h.Y[i], h.ldy[i]);
+                           h.bias ? h.bias[i] : nullptr, h.Y[i], h.ldy[i], h.post ? h.post[i].activation : DT_ACT_NONE,
+                           h.post ? h.post[i].gate : nullptr, h.post ? h.post[i].residual : nullptr,
+                           h.post ? h.post[i].ld_residual : 0);
         dt_status st = launch_status();
         if (st != DT_OK) return st;
         if (h.wants_epi(i)) {
@@ -1029,7 +1150,21 @@ DT_EXPORT dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K
                                           uint32_t flags) {
   using namespace dt;
   (void)flags;
-  const HostGroup h{M, K, X, ldx, W, n_weights, bias, Y, ldy, epi};
+  const HostGroup h{M, K, X, ldx, W, n_weights, bias, Y, ldy, epi, nullptr};
+  dt_status st = validate_group(h);
+  if (st != DT_OK) return st;
+  if (M == 0) return DT_OK;
+  if (!device_ok()) return DT_NO_KERNEL;
+  return run_group(as_stream(stream), h);
+}
+
+DT_EXPORT dt_status dt_dense_qx_post_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,
+                                         const dt_qx_weight* W, int32_t n_weights, const uint16_t* const* bias,
+                                         uint16_t* const* Y, const int64_t* ldy, const dt_dense_post* post,
+                                         uint32_t flags) {
+  using namespace dt;
+  (void)flags;
+  const HostGroup h{M, K, X, ldx, W, n_weights, bias, Y, ldy, nullptr, post};
   dt_status st = validate_group(h);
   if (st != DT_OK) return st;
   if (M == 0) return DT_OK;
@@ -1047,7 +1182,7 @@ DT_EXPORT dt_status dt_dense_qx_grouped_f16(dt_stream stream, int32_t n_groups, 
   int n = 0;
   for (int i = 0; i < n_groups; i++) {
     const dt_dense_group& d = groups[i];
-    const HostGroup h{d.M, d.K, d.X, d.ldx, d.W, d.n_weights, d.bias, d.Y, d.ldy, d.epi};
+    const HostGroup h{d.M, d.K, d.X, d.ldx, d.W, d.n_weights, d.bias, d.Y, d.ldy, d.epi, nullptr};
     dt_status st = validate_group(h);
     if (st != DT_OK) return st;
     if (h.M > 0) hs[n++] = h;

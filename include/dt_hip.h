@@ -150,6 +150,35 @@ dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K, const ui
                                 uint32_t flags);
 
 /*
+ * Dense followed by the elementwise tail of the feed-forward and residual paths
+ * of a transformer block, applied in the GEMM epilogue in this order, each step
+ * rounding to fp16 as the separate ops do:
+ *   activation : DT_ACT_GELU_TANH  linear1(x).GELU(approximate: .tanh)  (Models/Flux1.swift:133-135, Models/Wan.swift:52-53)
+ *                DT_ACT_SWISH      fc0(x).swish()                       (Models/Flux1.swift:122-123)
+ *   gate       : [N_i] fp16, multiplies every output row ((xOut .* xChunks[2]), Models/Flux1.swift:246-250)
+ *   residual   : fp32 [M, N_i] with row stride ld_residual, updated in place:
+ *                residual += float(result)  (x + (...).to(of: x), Models/Flux1.swift:250, 275-283)
+ * post: HOST array of n_weights entries (NULL = plain dt_dense_qx_f16).  Y[i] may
+ * be NULL when post[i].residual is given (the result is only accumulated).
+ * Concurrent calls must not share a residual tensor.
+ */
+#define DT_ACT_NONE 0
+#define DT_ACT_GELU_TANH 1
+#define DT_ACT_SWISH 2
+
+typedef struct {
+  int32_t activation;
+  const uint16_t* gate;
+  float* residual;
+  int64_t ld_residual;
+} dt_dense_post;
+
+dt_status dt_dense_qx_post_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,
+                               const dt_qx_weight* W, int32_t n_weights, const uint16_t* const* bias,
+                               uint16_t* const* Y, const int64_t* ldy, const dt_dense_post* post,
+                               uint32_t flags);
+
+/*
  * Several independent Dense problems (each an X with its weights, arguments as
  * for dt_dense_qx_heads_f16) enqueued together.  The context (text) and image
  * streams of a joint block apply different weights to different token sets

@@ -338,3 +338,27 @@ def synth_qx_weight(rng, N, K, qbits, nib, std=0.02):
     palettes = (rng.standard_normal((nblocks, 1 << qbits)) * std).astype(np.float16)
     idx = rng.integers(0, 1 << qbits, size=count, dtype=np.uint8)
     return C.palettize_pack(qbits, nib, palettes, idx), palettes, idx
+
+
+# ---------------------------------------------------------------------------
+# Elementwise tails of the feed-forward / residual paths (numpy; fp16 in, fp16 out, computed in float32 as the
+# reference's elementwise ops do).  Pinned in tests/test_oracle_ops.py by float64 closed forms (erf-GELU bound,
+# gelu(x) - gelu(-x) = x, limits, sigmoid identity) and exact small cases of the residual update.  GELU(approximate: .tanh): Models/Flux1.swift:133-135; swish: :122-123;
+# gated residual x + (y .* gate).to(of: x): :246-250, 275-283.
+# ---------------------------------------------------------------------------
+
+def np_gelu_tanh16(y16: np.ndarray) -> np.ndarray:
+    x = y16.astype(np.float32)
+    u = np.float32(0.7978845608028654) * (x + np.float32(0.044715) * x * x * x)
+    return (np.float32(0.5) * x * (np.float32(1) + np.tanh(u))).astype(np.float16)
+
+
+def np_swish16(y16: np.ndarray) -> np.ndarray:
+    x = y16.astype(np.float32)
+    return (x / (np.float32(1) + np.exp(-x))).astype(np.float16)
+
+
+def np_gated_residual(res32: np.ndarray, y16: np.ndarray, gate16=None) -> np.ndarray:
+    """res + float32(fp16(y * gate)); gate broadcast over rows."""
+    y = y16 if gate16 is None else (y16.astype(np.float32) * gate16.astype(np.float32)[None, :]).astype(np.float16)
+    return (res32.astype(np.float32) + y.astype(np.float32)).astype(np.float32)

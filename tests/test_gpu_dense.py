@@ -303,3 +303,71 @@ def test_dense_grouped_empty_and_bad(dthip, oracle, torch_cuda):
     bad = dthip.QxTensor(w.data, 3, w.nib, w.shape)
     with pytest.raises(dthip.DtError):
         dthip.dense_grouped([dict(x=x1, weights=[w], biases=[None]), dict(x=x1, weights=[bad], biases=[None])])
+
+
+@pytest.mark.parametrize("M,N,K,q,nib", [(300, 512, 256, 6, 4096), (1100, 384, 128, 4, 512), (70, 100, 96, 6, 64), (257, 256, 192, 16, 0)])
+def test_dense_post_feed_forward_and_residual(dthip, oracle, torch_cuda, M, N, K, q, nib):
+    """Dense with the elementwise tails of the block's feed-forward / residual paths in the epilogue:
+    linear1(x).GELU(tanh), swish, and x + (y .* gate).to(of: x) into an fp32 residual stream (with and without keeping
+    the fp16 result), against the oracle's Dense followed by its numpy tails.  One fp16 ulp on the activations (the
+    device evaluates tanh / sigmoid through exp2 and an approximate reciprocal)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(M + N)
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    if q == 16:
+        Wh = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+        w, ref = dthip.QxTensor.from_f16(Wh), lambda b: oracle.C.dense(X, Wh, b)
+    else:
+        w, p = make_weight(dthip, oracle, rng, N, K, q, nib, std=0.05)
+        ref = lambda b: oracle.C.dense_qx(X, p, q, nib, N, b)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float16)
+    gate = (1 + 0.3 * rng.standard_normal(N)).astype(np.float16)
+    res0 = rng.standard_normal((M, N)).astype(np.float32)
+    y = ref(bias)
+    xd, bd, gd = to_dev(torch, X), to_dev(torch, bias), to_dev(torch, gate)
+    print("dense post", M, N, K, q, flush=True)
+
+    def ulps(a, b):
+        ai, bi = a.view(np.int16).astype(np.int32), b.view(np.int16).astype(np.int32)
+        ai = np.where(ai < 0, -32768 - ai, ai)
+        bi = np.where(bi < 0, -32768 - bi, bi)
+        return np.abs(ai - bi).max()
+
+    # GELU / swish on two projections sharing x, plain third
+    outs = dthip.dense_post(xd, [w, w, w], [bd, bd, bd], [dthip.DensePost(dthip.ACT_GELU_TANH), dthip.DensePost(dthip.ACT_SWISH), None])
+    plain = dthip.dense_multi(xd, [w], [bd])[0]
+    assert torch.equal(outs[2], plain)
+    mx, rr = oracle.err_stats(plain.cpu().numpy(), y)
+    assert mx <= MAX_ABS and rr <= 2 * REL_RMS
+    y_dev = plain.cpu().numpy()              # tails are checked on the device's own Dense result: exact op-by-op semantics
+    assert ulps(outs[0].cpu().numpy(), oracle.np_gelu_tanh16(y_dev)) <= 1
+    assert ulps(outs[1].cpu().numpy(), oracle.np_swish16(y_dev)) <= 1
+    # gated residual, fp16 result kept
+    res = torch.from_numpy(res0.copy()).cuda()
+    o = dthip.dense_post(xd, [w], [bd], [dthip.DensePost(gate=gd, residual=res)])[0]
+    want16 = (y_dev.astype(np.float32) * gate.astype(np.float32)[None, :]).astype(np.float16)
+    assert np.array_equal(o.cpu().numpy().view(np.uint16), want16.view(np.uint16))
+    assert np.array_equal(res.cpu().numpy(), oracle.np_gated_residual(res0, y_dev, gate))
+    # accumulate only (no fp16 output), no gate, GELU first; residual is a row-strided view
+    big = torch.zeros((M, N + 8), dtype=torch.float32, device="cuda")
+    view = big[:, 4:4 + N]
+    view.copy_(torch.from_numpy(res0))
+    o2 = dthip.dense_post(xd, [w], [bd], [dthip.DensePost(dthip.ACT_GELU_TANH, residual=view, keep_output=False)])[0]
+    assert o2 is None
+    got = view.cpu().numpy()
+    want = oracle.np_gated_residual(res0, oracle.np_gelu_tanh16(y_dev))
+    assert np.max(np.abs(got - want)) <= 2.0 ** -10 * np.maximum(1, np.abs(y_dev.astype(np.float32))).max()
+    assert float(big[:, :4].abs().max()) == 0 and float(big[:, 4 + N:].abs().max()) == 0
+
+
+def test_dense_post_bad_args(dthip, oracle, torch_cuda):
+    torch = torch_cuda
+    rng = np.random.default_rng(9)
+    w, _ = make_weight(dthip, oracle, rng, 64, 64, 6, 64)
+    x = to_dev(torch, rng.standard_normal((4, 64)).astype(np.float16))
+    with pytest.raises(dthip.DtError):
+        dthip.dense_post(x, [w], [None], [dthip.DensePost(activation=7)])
+    with pytest.raises((ValueError, TypeError)):
+        dthip.dense_post(x, [w], [None], [dthip.DensePost(residual=torch.zeros((4, 64), dtype=torch.float16, device="cuda"))])
+    with pytest.raises(ValueError):
+        dthip.dense_post(x, [w], [None], [dthip.DensePost(gate=torch.zeros(3, dtype=torch.float16, device="cuda"))])

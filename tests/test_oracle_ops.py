@@ -243,3 +243,36 @@ def test_instruction_counts(oracle):
     # DenseInstructionCount = M*N*K, SDPA = B*H*(2D+5)*Sa*Sb
     assert oracle.C.dense_instruction_count(4608, 3072, 3072) == 4608 * 3072 * 3072
     assert oracle.C.sdpa_instruction_count(1, 24, 128, 4608, 4608) == 24 * 261 * 4608 * 4608
+
+
+def test_elementwise_tails_pinned(oracle):
+    """GELU(tanh), swish and the gated residual against what the mathematics fixes."""
+    import math
+    x = np.linspace(-8, 8, 4001).astype(np.float16)
+    g = oracle.np_gelu_tanh16(x).astype(np.float64)
+    xd = x.astype(np.float64)
+    # odd-part identity of any 0.5*x*(1+odd(x)) function: gelu(x) - gelu(-x) = x
+    assert np.max(np.abs((g - g[::-1]) - xd)) <= 2e-3 * (1 + np.abs(xd)).max()
+    # float64 statement of the same formula, rounded once
+    want = 0.5 * xd * (1 + np.tanh(math.sqrt(2 / math.pi) * (xd + 0.044715 * xd ** 3)))
+    assert np.array_equal(oracle.np_gelu_tanh16(x), want.astype(np.float16)) or \
+        np.max(np.abs(g - want)) <= np.finfo(np.float16).eps * np.maximum(1, np.abs(want)).max()
+    # the tanh form stays within 5e-4 + 0.5 % of the exact erf GELU it approximates, and has its limits
+    erf = np.vectorize(math.erf)
+    exact = 0.5 * xd * (1 + erf(xd / math.sqrt(2)))
+    assert np.max(np.abs(g - exact)) <= 3e-3
+    assert g[x == 0][0] == 0 and abs(g[-1] - 8) < 1e-2 and abs(g[0]) < 1e-3
+    # swish(x) = x * sigmoid(x); swish(x) + swish(-x) = x * tanh(x / 2)
+    s = oracle.np_swish16(x).astype(np.float64)
+    assert np.max(np.abs(s - xd / (1 + np.exp(-xd)))) <= 4e-3
+    assert np.max(np.abs((s + s[::-1]) - xd * np.tanh(xd / 2))) <= 8e-3
+    # gated residual: exact on values that need no rounding; gate broadcast over rows; fp16 rounding of the product
+    res = np.array([[1.0, 2.0], [3.0, 4.0]], np.float32)
+    y = np.array([[0.5, -1.0], [2.0, 0.25]], np.float16)
+    gate = np.array([2.0, 4.0], np.float16)
+    assert np.array_equal(oracle.np_gated_residual(res, y, gate), np.array([[2.0, -2.0], [7.0, 5.0]], np.float32))
+    assert np.array_equal(oracle.np_gated_residual(res, y), res + y.astype(np.float32))
+    y2 = np.array([[1.0009765625]], np.float16)            # 1 + 2^-10
+    g2 = np.array([1.0009765625], np.float16)
+    # (1 + 2^-10)^2 = 1 + 2^-9 + 2^-20 rounds to 1 + 2^-9 in fp16 before it reaches the fp32 stream
+    assert oracle.np_gated_residual(np.zeros((1, 1), np.float32), y2, g2)[0, 0] == np.float32(1 + 2.0 ** -9)
