@@ -286,3 +286,32 @@ def test_sdpa_flux_full_size_sampled(dthip, oracle, torch_cuda):
     vc = torch.from_numpy(f16(rng.standard_normal((1, 1, H, D)))).cuda().expand(B, S, H, D).contiguous()
     oc = dthip.ScaledDotProductAttention(scale=scale)(qd, kd, vc)
     assert float((oc.float() - vc.float()).abs().max()) <= 2e-3
+
+
+def test_sdpa_wan_full_size_sampled(dthip, oracle, torch_cuda):
+    """BASELINE's largest shape (1, 40 heads x 128, 32760 tokens; Q and K pre-scaled by D^-1/4 and scale 1, the
+    `.scale1` convention of Models/Wan.swift:95-103): sampled rows of two heads against the oracle, the
+    constant-V property over the whole output, and scale1 == scaleMerged on the sampled rows' neighbourhood."""
+    torch = torch_cuda
+    rng = np.random.default_rng(21)
+    B, S, H, D = 1, 32760, 40, 128
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    qd = torch.randn((B, S, H, D), device="cuda", generator=gen).half()
+    kd = torch.randn((B, S, H, D), device="cuda", generator=gen).half()
+    vd = torch.randn((B, S, H, D), device="cuda", generator=gen).half()
+    s4 = float(D) ** -0.25
+    q1, k1 = (qd.float() * s4).half(), (kd.float() * s4).half()
+    print("sdpa wan full size", flush=True)
+    got = dthip.ScaledDotProductAttention(scale=1.0)(q1, k1, vd)
+    rows = np.sort(rng.choice(S, size=16, replace=False))
+    rows[0], rows[-1] = 0, S - 1
+    rt = torch.from_numpy(rows).cuda()
+    for h in (0, 39):
+        want = oracle.C.sdpa(np.ascontiguousarray(q1[:, rt, h:h + 1].cpu().numpy()), np.ascontiguousarray(k1[:, :, h:h + 1].cpu().numpy()),
+                             np.ascontiguousarray(vd[:, :, h:h + 1].cpu().numpy()), 1.0)
+        mx, rr = oracle.err_stats(got[:, rt, h:h + 1].cpu().numpy(), want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (h, mx, rr)
+    del got
+    vc = torch.randn((1, 1, H, D), device="cuda", generator=gen).half().expand(B, S, H, D).contiguous()
+    oc = dthip.ScaledDotProductAttention(scale=1.0)(q1, k1, vc)
+    assert float((oc.float() - vc.float()).abs().max()) <= 2e-3

@@ -371,3 +371,28 @@ def test_dense_post_bad_args(dthip, oracle, torch_cuda):
         dthip.dense_post(x, [w], [None], [dthip.DensePost(residual=torch.zeros((4, 64), dtype=torch.float16, device="cuda"))])
     with pytest.raises(ValueError):
         dthip.dense_post(x, [w], [None], [dthip.DensePost(gate=torch.zeros(3, dtype=torch.float16, device="cuda"))])
+
+
+def test_dense_wan_full_size_sampled(dthip, oracle, torch_cuda):
+    """BASELINE's largest Dense (M 32760, 5120 -> 5120, q5p with 1024-element blocks: five palette blocks per weight
+    row): a sample of rows against the oracle, plus linearity Y(2x) == 2 Y(x)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(15)
+    M, K, N, q, nib = 32760, 5120, 5120, 5, 1024
+    w, p = make_weight(dthip, oracle, rng, N, K, q, nib)
+    bias = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    gen = torch.Generator(device="cuda").manual_seed(15)
+    xd = torch.randn((M, K), device="cuda", generator=gen).half()
+    print("dense wan full size", flush=True)
+    out = dthip.dense_multi(xd, [w], [to_dev(torch, bias)])[0]
+    rows = np.sort(rng.choice(M, size=16, replace=False))
+    rows[0], rows[-1] = 0, M - 1
+    rt = torch.from_numpy(rows).cuda()
+    want = oracle.C.dense_qx(np.ascontiguousarray(xd[rt].cpu().numpy()), p, q, nib, N, bias)
+    mx, rr = oracle.err_stats(out[rt].cpu().numpy(), want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+    a = dthip.dense_multi(xd, [w], [None])[0]
+    b = dthip.dense_multi(xd * 2, [w], [None])[0]
+    normal = a.abs() >= 2.0 ** -13
+    assert torch.equal((a * 2)[normal], b[normal])
+    assert float((a.float() * 2 - b.float()).abs().max()) <= 2.0 ** -23
