@@ -307,9 +307,6 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // pair slot (pairs past the end re-read the last one, harmlessly).
   auto issue_pair_part = [&](half_t* xs, half_t* wp, int q, int i) {
     if (q > last_pair) q = last_pair;
-#ifdef DT_EXP_NODMA
-    if (q > 0) return;
-#endif
     const int64_t kb = (int64_t)q * (4 * BK);  // byte offset of the pair inside a row
     if (i < AP) {
       load_to_lds_16(xbase + kb, a_off[i], lds_address(xs) + (uint32_t)((wave_u * AP + i) * 1024));
@@ -423,18 +420,12 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   half8_t fw[2][TN], fx[2][TM];
   // par: tile of the pair (0/1), ks: k-step of the tile, stage: ring stage of the unpacked weights
   auto read_w = [&](int buf, int i, const half_t* wp, int par, int stage, int ks) {
-#ifdef DT_EXP_NOREAD
-    if (buf >= 0) return;
-#endif
     if constexpr (MODE == kPlainF16)
       fw[buf][i] = *reinterpret_cast<const half8_t*>(wp + (w_lane ^ ((4 * par + 2 * ks) << 3)) + i * 32 * PROW);
     else
       fw[buf][i] = *reinterpret_cast<const half8_t*>(Bs + stage * B_STAGE + lds_chunk(wrow + i * 32, 2 * ks + hi));
   };
   auto read_x = [&](int buf, int j, const half_t* xs, int par, int ks) {
-#ifdef DT_EXP_NOREAD
-    if (buf >= 0) return;
-#endif
     fx[buf][j] = *reinterpret_cast<const half8_t*>(xs + (x_lane ^ ((4 * par + 2 * ks) << 3)) + j * 32 * PROW);
   };
   auto mfma = [&](int buf, int i, int j) {
@@ -558,15 +549,10 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       for (int k = m * n1 / NM; k < (m + 1) * n1 / NM; k++) place(k, ns1, read1, stage1);
     }
     __builtin_amdgcn_sched_barrier(0);
-#ifndef DT_EXP_NOWAIT
     if (par == 0)
       __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
     else
       __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
-#endif
-#ifdef DT_EXP_NOBAR
-    if (par == 1)
-#endif
     __syncthreads();
     const int s = s_cur;
     s_cur = s_nxt;

@@ -301,16 +301,6 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
 
   // online softmax of tile t (per query column, statistics in fp32): sacc -> pf
   auto softmax_phase = [&](int t) __attribute__((always_inline)) {
-#ifdef DT_EXP_NOSOFTMAX
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-      for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) pf[kb][tt][e] = (half_t)(sacc[kb][8 * tt + e] * 1e-3f);
-    l_run = 1.f;
-    return;
-#endif
     const int rem = (int)(Skv - (int64_t)t * BKV);  // keys left, this tile included
     const bool ragged = rem < BKV;
     if (PREMUL || ragged) {
@@ -352,13 +342,7 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       for (int tt = 0; tt < 2; tt++)
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-#if defined(DT_EXP_NOEXP)
-          const float p = __builtin_fmaf(sacc[kb][8 * tt + e], c, -mc) * 1e-3f;
-#elif defined(DT_EXP_EXPONLY)
-          const float p = fast_exp2(sacc[kb][8 * tt + e]);
-#else
           const float p = fast_exp2(__builtin_fmaf(sacc[kb][8 * tt + e], c, -mc));
-#endif
           psum += p;
           pf[kb][tt][e] = (half_t)p;
         }
@@ -412,15 +396,9 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   // interval t: K(t) is in k_cur, V(t-1) in v_prev; K(t+1) goes to k_next, V(t) to v_cur
   auto interval = [&](int t, const unsigned char* k_cur, unsigned char* k_next, const unsigned char* v_prev,
                       unsigned char* v_cur) __attribute__((always_inline)) {
-#ifndef DT_EXP_NODMA
     if (t + 1 < n_tiles) issue_k(k_next);
     if (t < n_tiles) issue_v(v_cur);
-#endif
-#ifdef DT_EXP_NOSKEW
-    if (true) {
-#else
     if (!second) {
-#endif
       if (t > 0) pv_phase(v_prev);
       if (t < n_tiles) {
         s_phase(k_cur);
@@ -433,9 +411,7 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       }
       if (t < n_tiles) s_phase(k_cur);
     }
-#ifndef DT_EXP_NOWAIT
     __builtin_amdgcn_s_waitcnt(0x0f70);
-#endif
     __syncthreads();
   };
   for (int t = 0; t <= n_tiles; t += 2) {
