@@ -1,15 +1,15 @@
 // K1: Dense over palettized weights, Y = X W^T (+ bias), for gfx950.
 //
-// The packed weight never exists dequantized in memory: per K-tile each thread
-// pulls one 32-index granule (Q dwords) of a weight row into registers,
-// unpacks it with constant shifts, looks the fp16 values up in the palettes
-// held in LDS, and writes the fp16 row slice into the LDS B tile that
-// v_mfma_f32_32x32x16_f16 then consumes.  fp32 accumulation, one rounding.
+// The packed weight never exists dequantized in memory: per K-tile two threads
+// per weight row each pull half of a 32-index granule into registers, unpack
+// it, look the fp16 values up in palettes held in LDS, and write the fp16 row
+// slice into an LDS ring that v_mfma_f32_32x32x16_f16 then consumes; X (and a
+// plain fp16 weight) goes from memory straight into LDS.  fp32 accumulation,
+// one rounding to fp16, optional fused tails (per-head RMSNorm + RoPE, or
+// activation / gate / fp32 residual).
 //
-// Tile: BM x BN outputs per 256-thread workgroup (4 waves as 2 x 2), BK = 32.
-// LDS is double-buffered; the global loads of tile t+1 are issued before the
-// MFMAs of tile t and its unpack/lookup runs after them, so one barrier per
-// K-tile and the unpack VALU/LDS work overlaps the matrix pipe.
+// Tile: BM x BN outputs per 512-thread workgroup (8 waves, two per SIMD, each
+// a BN/2 x BM/4 slice), K-tiles of 32 processed in pairs; one barrier per K-tile.
 #include <numeric>
 
 #include "dt_common.h"
@@ -21,7 +21,6 @@ namespace dt {
 constexpr int kMaxWeights = 8;
 constexpr int kMaxGroups = 4;
 constexpr int BK = 32;
-constexpr int LDS_ROW = BK + 8;  // halfs; 80-byte rows keep 16-byte LDS accesses of 8 consecutive rows on distinct banks
 constexpr int kPalLdsBytes = 32768;
 
 enum PalMode : int {
@@ -124,15 +123,15 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
   return (uint32_t)half_to_bits((half_t)a) | ((uint32_t)half_to_bits((half_t)b) << 16);
 }
 
-// 512 threads = 8 waves, two per SIMD.  Every thread stages two 16-byte chunks
-// of the X tile and unpacks / looks up half a granule (16 weights) of one W
-// row per K-tile, so the LDS instructions -- which a single wave can only
-// issue every few tens of clocks -- are spread evenly over all eight waves.
-// Waves w and w+4 share a SIMD and run the two halves of an iteration in
-// opposite order, so one of them is always feeding the matrix pipe.  All
-// eight run MFMAs on a (BN/2) x (BM/4) slice.  The accumulators are held
-// transposed (rows = output features n, columns = tokens m) so that each lane
-// ends up with runs of consecutive n for one token: 16-byte stores.
+// 512 threads = 8 waves, two per SIMD, all eight running MFMAs on a (BN/2) x
+// (BM/4) slice.  Every thread issues its share of the memory -> LDS transfer of
+// X and unpacks / looks up half a granule (16 weights) of one W row per
+// K-tile, so the LDS instructions -- the scarce resource: a wave can issue one
+// only every few tens of clocks and the CU's LDS pipe handles one every 2-4 --
+// are spread evenly over all waves and between their MFMAs.  The accumulators
+// are held transposed (rows = output features n, columns = tokens m) so that
+// each lane ends up with runs of consecutive n for one token: 16-byte stores.
+// POST selects the epilogue with the elementwise tail.
 template <int Q, int BM, int BN, int MODE, bool POST>
 __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   constexpr int WN = BN / 2, WM = BM / 4;   // per-wave slice: WN features x WM tokens
@@ -147,8 +146,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   static_assert(BM % 128 == 0 && BN % 128 == 0 && BN <= 256, "tile");
 
   // X (and a plain fp16 W) lives in two pair slots, each holding two K-tiles
-  // as [rows][64 halfs]; the slots are separate arrays so that reads of one
-  // are known not to touch the other while a load into it is in flight.
+  // as [rows][64 halfs]: one is read while the next pair is in flight into the other.
   __shared__ __attribute__((aligned(1024))) half_t XsA[BM * PROW];
   __shared__ __attribute__((aligned(1024))) half_t XsB[BM * PROW];
   __shared__ __attribute__((aligned(1024))) half_t WpA[MODE == kPlainF16 ? BN * PROW : 8];
@@ -160,7 +158,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const bool second = wave >= 4;     // stages first, then runs its MFMAs; unpacks weights 16..31 of its granule
+  const bool second = wave >= 4;     // unpacks weights 16..31 of its row's granule (waves 0-3: weights 0..15)
   const int lt = tid & 255;
   const int wn = wave & 1, wm = (wave >> 1) & 1 | ((wave >> 2) << 1);  // waves w and w+4 share a SIMD and take different m slices
 
@@ -371,10 +369,9 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     else if constexpr (MODE != kPlainF16)
       la[j] = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(Pal) + la[j]);
   };
-  // Written as assembly: the compiler makes every LDS store it knows of wait
-  // for all memory -> LDS transfers in flight, which would stall the even
-  // iterations until the next pair has landed.  The closing s_waitcnt of an
-  // iteration covers these stores.
+  // Written as assembly, like the transfers: the closing s_waitcnt of an
+  // iteration covers these stores, and the compiler has no reason to order
+  // them against anything else.
   const uint32_t w_dst = lds_address(Bs) + 2u * (uint32_t)lds_chunk(b_row, second ? 2 : 0);
   auto write_weights = [&](int stage, int h) {
     if constexpr (MODE != kPlainF16) {
@@ -480,8 +477,9 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       }
     }
     IdxSet& R = WS[par];
-    // the wait for the indices comes here, before the transfer goes out: a
-    // wait with the transfer outstanding would last until it lands
+    // the wait for the indices comes here, before the transfer goes out: vector
+    // memory loads return in order, so a wait with the transfer outstanding
+    // would last until it lands
     touch(R);
     if (par) issue_idx(WS[0]);  // tile t+3
     const half_t* xs_n = par == 0 ? xs : xs_other;  // fragments of tile t+1, k-step 0

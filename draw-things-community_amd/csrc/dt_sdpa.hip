@@ -2,7 +2,8 @@
 //
 // One 512-thread workgroup (8 waves, two per SIMD) owns 256 query rows of one
 // (batch, head); each wave owns 32 of them.  K/V arrive in tiles of 64 keys,
-// staged row-major through LDS (double-buffered, one barrier per tile).
+// transferred from memory straight into LDS, row-major (double-buffered, one
+// barrier per tile).
 //
 // Everything is computed transposed so that the query index is the MFMA
 // column (lane & 31) in every stage:
@@ -58,9 +59,8 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   constexpr int KS = DP / 16;                  // MFMA k-steps over the head dimension
   static_assert(LOADS >= 1, "tile");
 
-  // Two stages each for K and V, as separate arrays: a tile is read from one
-  // while the next is in flight into the other, and only for distinct arrays
-  // does the compiler know that those reads need not wait for the transfer.
+  // Two stages each for K and V: a tile is read from one while the next is in
+  // flight into the other.
   __shared__ __attribute__((aligned(1024))) unsigned char Ks0[TILE_B];
   __shared__ __attribute__((aligned(1024))) unsigned char Ks1[TILE_B];
   __shared__ __attribute__((aligned(1024))) unsigned char Vs0[TILE_B];
