@@ -81,16 +81,23 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
 }
 // source = uniform 64-bit base + 32-bit per-lane byte offset
 __device__ __forceinline__ void load_to_lds_16(const void* gbase, uint32_t voff, uint32_t lds_base) {
+  // the base must sit in scalar registers whatever the control flow around the call made of it
+  const uint64_t gb = (uint64_t)(uintptr_t)gbase;
+  // (the builtin returns a signed int: widen through uint32_t, or bit 31 of the low half smears over the high half)
+  const uint64_t gu = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)gb) |
+                      ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(gb >> 32)) << 32);
+  lds_base = (uint32_t)__builtin_amdgcn_readfirstlane(lds_base);
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
       "s_nop 0\n\t"
       "global_load_lds_dwordx4 %1, %2"
       :
-      : "s"(lds_base), "v"(voff), "s"(gbase)
+      : "s"(lds_base), "v"(voff), "s"(gu)
       : "memory");
 }
 // source = per-lane 64-bit address
 __device__ __forceinline__ void load_to_lds_16(const void* gptr, uint32_t lds_base) {
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
       "s_nop 0\n\t"
