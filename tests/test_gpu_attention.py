@@ -315,3 +315,59 @@ def test_sdpa_wan_full_size_sampled(dthip, oracle, torch_cuda):
     vc = torch.randn((1, 1, H, D), device="cuda", generator=gen).half().expand(B, S, H, D).contiguous()
     oc = dthip.ScaledDotProductAttention(scale=1.0)(q1, k1, vc)
     assert float((oc.float() - vc.float()).abs().max()) <= 2e-3
+
+
+def test_block_step_replays_as_hip_graph(dthip, oracle, torch_cuda):
+    """The three launches of a joint block (grouped QKV Dense with the fused norm / RoPE epilogue, attention, grouped
+    out-projection) captured as one HIP graph: every replay, with eager runs and synchronisations in between,
+    reproduces the eager result bit for bit (no call on this path allocates or clears memory behind the capture)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(33)
+    T, HW, H, D = 64, 320, 2, 128
+    C, S = H * D, 64 + 320
+    def mk():
+        packed, _, _ = oracle.synth_qx_weight(rng, C, C, 6, 4096, 0.05)
+        return dthip.QxTensor.from_packed(packed, 6, 4096, (C, C))
+    w = {n: mk() for n in ("c_q", "c_k", "c_v", "x_q", "x_k", "x_v", "c_o", "x_o")}
+    f = lambda shape, s=1.0: to_dev(torch, (rng.standard_normal(shape) * s).astype(np.float16))
+    ctx, img = f((T, C)), f((HW, C))
+    gam = {n: f((D,), 0.05) + 1 for n in ("c_q", "c_k", "x_q", "x_k")}
+    rot = to_dev(torch, dthip.Flux1RotaryPositionEmbedding(16, 20, T, channels=D).astype(np.float16))
+    qkv = torch.zeros((S, 3, H, D), dtype=torch.float16, device="cuda")
+    att = torch.zeros((1, S, H, D), dtype=torch.float16, device="cuda")
+    out_c = torch.zeros((T, C), dtype=torch.float16, device="cuda")
+    out_x = torch.zeros((HW, C), dtype=torch.float16, device="cuda")
+    qkv2 = qkv.view(S, 3 * C)
+    views = lambda lo, hi: [qkv2[lo:hi, i * C:(i + 1) * C] for i in range(3)]
+    epi = lambda a, b, pos: [dthip.HeadEpilogue(gam[a], rot, pos, 1e-6, D), dthip.HeadEpilogue(gam[b], rot, pos, 1e-6, D), None]
+    att2 = att.view(S, C)
+
+    def step():
+        dthip.dense_grouped([
+            dict(x=img, weights=[w["x_q"], w["x_k"], w["x_v"]], biases=[None] * 3, outs=views(T, S), epilogues=epi("x_q", "x_k", T)),
+            dict(x=ctx, weights=[w["c_q"], w["c_k"], w["c_v"]], biases=[None] * 3, outs=views(0, T), epilogues=epi("c_q", "c_k", 0))])
+        dthip.sdpa_segments([qkv[:, 0].unsqueeze(0)], [qkv[:, 1].unsqueeze(0)], [qkv[:, 2].unsqueeze(0)], 1 / np.sqrt(D), out=att)
+        dthip.dense_grouped([dict(x=att2[T:], weights=[w["x_o"]], biases=[None], outs=[out_x]),
+                             dict(x=att2[:T], weights=[w["c_o"]], biases=[None], outs=[out_c])])
+
+    print("block step as hip graph", flush=True)
+    step()
+    torch.cuda.synchronize()
+    want = (out_x.clone(), out_c.clone(), att.clone())
+    assert float(want[0].abs().max()) > 0
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for _ in range(4):
+        out_x.zero_(); out_c.zero_(); att.zero_(); qkv.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a_, b_ in zip((out_x, out_c, att), want):
+            assert torch.equal(a_, b_)
+        step()
+        torch.cuda.synchronize()
