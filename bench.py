@@ -199,7 +199,7 @@ def main():
         "sdpa_S4608": time_kernel(k_sdpa, it),
         "dense_out_2x": time_kernel(k_out, it),
     }
-    # BASELINE "palettized Dense alone" shape: M = 4608, 3072 -> 9216 (three weights) and 3072 -> 3072
+    # the "palettized Dense alone" shape of the headline benchmark: M = 4608, 3072 -> 9216 (three weights) and 3072 -> 3072
     x_all = f16((S, C))
     y3 = [torch.empty((S, C), dtype=torch.float16, device=dev) for _ in range(3)]
     ms["dense_qkv_M4608_N9216"] = time_kernel(

@@ -331,7 +331,7 @@ def err_stats(got, want):
 
 
 def synth_qx_weight(rng, N, K, qbits, nib, std=0.02):
-    """BASELINE-style synthetic palettized weight: per-block N(0, std) fp16
+    """Synthetic palettized weight of the benchmark kind: per-block N(0, std) fp16
     palettes and uniform indices.  Returns (packed uint8, palettes, idx)."""
     count = N * K
     nblocks = (count + nib - 1) // nib

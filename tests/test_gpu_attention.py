@@ -265,7 +265,7 @@ def test_sdpa_rejects_bad_arguments(dthip, torch_cuda):
 
 
 def test_sdpa_flux_full_size_sampled(dthip, oracle, torch_cuda):
-    """BASELINE shape (1, 24 heads x 128, 512 text + 4096 image tokens): sampled rows of two heads against
+    """Headline benchmark shape (1, 24 heads x 128, 512 text + 4096 image tokens): sampled rows of two heads against
     the oracle, and the constant-V property over the whole output."""
     torch = torch_cuda
     rng = np.random.default_rng(9)
@@ -289,7 +289,7 @@ def test_sdpa_flux_full_size_sampled(dthip, oracle, torch_cuda):
 
 
 def test_sdpa_wan_full_size_sampled(dthip, oracle, torch_cuda):
-    """BASELINE's largest shape (1, 40 heads x 128, 32760 tokens; Q and K pre-scaled by D^-1/4 and scale 1, the
+    """The largest benchmark shape (1, 40 heads x 128, 32760 tokens; Q and K pre-scaled by D^-1/4 and scale 1, the
     `.scale1` convention of Models/Wan.swift:95-103): sampled rows of two heads against the oracle, the
     constant-V property over the whole output, and scale1 == scaleMerged on the sampled rows' neighbourhood."""
     torch = torch_cuda

@@ -172,7 +172,7 @@ def test_dense_rejects_bad_arguments(dthip, torch_cuda):
 
 
 def test_dense_flux_qkv_full_size_sampled(dthip, oracle, torch_cuda):
-    """BASELINE shape (M 4608, K 3072, three N 3072 q6p weights in one launch): a sample of rows
+    """Headline benchmark shape (M 4608, K 3072, three N 3072 q6p weights in one launch): a sample of rows
     against the oracle, plus linearity Y(2x) == 2 Y(x) (power-of-two scaling is exact in fp32 and in normal fp16)."""
     torch = torch_cuda
     rng = np.random.default_rng(14)
@@ -374,7 +374,7 @@ def test_dense_post_bad_args(dthip, oracle, torch_cuda):
 
 
 def test_dense_wan_full_size_sampled(dthip, oracle, torch_cuda):
-    """BASELINE's largest Dense (M 32760, 5120 -> 5120, q5p with 1024-element blocks: five palette blocks per weight
+    """The largest benchmark Dense (M 32760, 5120 -> 5120, q5p with 1024-element blocks: five palette blocks per weight
     row): a sample of rows against the oracle, plus linearity Y(2x) == 2 Y(x)."""
     torch = torch_cuda
     rng = np.random.default_rng(15)
