@@ -263,21 +263,21 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       reinterpret_cast<uint32_t*>(Pal)[i] = src[e];
     }
   }
-  // kPalRow: Pal is a table [64-row group][entry][row % 64] of fp16, so the 64
-  // lanes of a wave (64 consecutive rows, one entry each) read 64 consecutive
-  // halfs of some entry rows: two lanes share a bank, nothing worse.  Each of a
-  // row's two threads keeps half of the row's column current.
-  const int pal_col = (b_row >> 6) * (128 << Q) + (b_row & 63) * 2;  // byte offset of this row's column
+  // kPalRow: Pal is a table [128-row group][entry][row % 64][row / 64 % 2] of
+  // fp16: rows r and r + 64 share a dword, so the 64 lanes of a wave (64
+  // consecutive rows, one entry each) hit 64 different banks whatever entries
+  // they ask for.  Each of a row's two threads keeps half of the row's column current.
+  const int pal_col = (b_row >> 7) * (256 << Q) + (b_row & 63) * 4 + ((b_row >> 6) & 1) * 2;  // byte offset of this row's column
   auto fill_pal_column = [&](int64_t blk) {
     constexpr int ND = (1 << Q) / 4;  // dwords of palette per thread
     const uint32_t* src =
         reinterpret_cast<const uint32_t*>(w.data + palette_offset(lay, blk)) + (second ? ND : 0);
-    char* dst = reinterpret_cast<char*>(Pal) + pal_col + (second ? (64 << Q) : 0);
+    char* dst = reinterpret_cast<char*>(Pal) + pal_col + (second ? (128 << Q) : 0);
 #pragma unroll
     for (int d = 0; d < ND; d++) {
       const uint32_t v = src[d];
-      *reinterpret_cast<uint16_t*>(dst + (2 * d) * 128) = (uint16_t)v;
-      *reinterpret_cast<uint16_t*>(dst + (2 * d + 1) * 128) = (uint16_t)(v >> 16);
+      *reinterpret_cast<uint16_t*>(dst + (2 * d) * 256) = (uint16_t)v;
+      *reinterpret_cast<uint16_t*>(dst + (2 * d + 1) * 256) = (uint16_t)(v >> 16);
     }
   };
   int gn_row = n0 + b_row;  // this thread's weight row
@@ -360,7 +360,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       }
 #pragma unroll
       for (int j = 4 * p; j < 4 * p + 4; j++)
-        la[j] = own_index_at<Q, HW, (MODE == kPalRow ? 7 : 1)>(be, j, pal_base);
+        la[j] = own_index_at<Q, HW, (MODE == kPalRow ? 8 : 1)>(be, j, pal_base);
     }
   };
   auto lookup = [&](int j) {
