@@ -62,7 +62,8 @@ class _HeadEpilogue(ctypes.Structure):
 
 class _DensePost(ctypes.Structure):
     _fields_ = [("activation", ctypes.c_int32), ("gate", ctypes.c_void_p), ("residual", ctypes.c_void_p),
-                ("ld_residual", ctypes.c_int64)]
+                ("ld_residual", ctypes.c_int64), ("scale", ctypes.c_float), ("addend", ctypes.c_void_p),
+                ("ld_addend", ctypes.c_int64)]
 
 
 class _DenseGroup(ctypes.Structure):
@@ -352,12 +353,15 @@ ACT_NONE, ACT_GELU_TANH, ACT_SWISH = 0, 1, 2
 
 
 class DensePost:
-    """Elementwise tail of one projection: activation (ACT_*), per-feature fp16 gate [N], fp32 residual [M, N] that the
+    """Elementwise tail of one projection, in this order: scalar `scale`, fp16 `addend` [M, N] (the low-rank branch of a
+    LoRADense, Models/LoRA.swift:117-140), activation (ACT_*), per-feature fp16 gate [N], fp32 residual [M, N] that the
     result is accumulated into (`x + (y .* gate).to(of: x)`, Models/Flux1.swift:250).  With `residual` given and
     `keep_output=False` the fp16 result itself is not written."""
 
-    def __init__(self, activation: int = ACT_NONE, gate=None, residual=None, keep_output: bool = True):
+    def __init__(self, activation: int = ACT_NONE, gate=None, residual=None, keep_output: bool = True,
+                 scale: float = 1.0, addend=None):
         self.activation, self.gate, self.residual, self.keep_output = activation, gate, residual, keep_output
+        self.scale, self.addend = scale, addend
 
 
 def dense_post(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]], posts: Sequence[Optional[DensePost]],
@@ -370,7 +374,7 @@ def dense_post(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]
     P = (_DensePost * n)()
     for i, p in enumerate(posts):
         if p is None:
-            P[i] = _DensePost(ACT_NONE, None, None, 0)
+            P[i] = _DensePost(ACT_NONE, None, None, 0, 1.0, None, 0)
             continue
         N = weights[i].shape[0]
         if p.gate is not None and (_f16_cuda(p.gate, "gate").numel() != N or not p.gate.is_contiguous()):
@@ -387,7 +391,14 @@ def dense_post(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]
             if not p.keep_output:
                 Y[i] = None
                 outs[i] = None
-        P[i] = _DensePost(p.activation, None if p.gate is None else p.gate.data_ptr(), rp, ldr)
+        ap, lda = None, 0
+        if p.addend is not None:
+            a2 = _f16_cuda(p.addend, "addend")
+            a2 = a2.reshape(-1, N) if a2.dim() != 2 else a2
+            if a2.shape != (M, N) or a2.stride(1) != 1 or a2.data_ptr() != p.addend.data_ptr():
+                raise ValueError("addend must be an [M, N] view with contiguous rows")
+            ap, lda = a2.data_ptr(), a2.stride(0)
+        P[i] = _DensePost(p.activation, None if p.gate is None else p.gate.data_ptr(), rp, ldr, float(p.scale), ap, lda)
     st = lib().dt_dense_qx_post_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, P, flags)
     _check("dt_dense_qx_post_f16", st)
     lead = tuple(x.shape[:-1])
@@ -424,6 +435,67 @@ class Dense:
             raise ValueError(f"Dense {self.name!r}: weight has {self.weight.shape[0]} rows, count is {self.count}")
         b = None if self.noBias else self.bias
         return dense_multi(x, [self.weight], [b], flags=self.flags, stream=stream)[0]
+
+
+class LoRANetworkConfiguration:
+    """rank / scale / highPrecision of the low-rank branch (Models/LoRA.swift:4-22)."""
+
+    def __init__(self, rank: int, scale: float = 1.0, highPrecision: bool = False):
+        self.rank, self.scale, self.highPrecision = rank, scale, highPrecision
+
+
+class LoRADense:
+    """LoRADense(count:configuration:noBias:flags:name:) -- dense(x) + up(scale * down(x)) with the palettized base
+    left packed and the fp16 low-rank pair applied beside it (Models/LoRA.swift:85-142; running the LoRA separately
+    is the preferred mode for quantized models, Models/UNetProtocol.swift:696-697).  Three launches of the Dense
+    kernel: down (with the scale in its epilogue), up, then the base projection whose epilogue adds the branch; every
+    intermediate is rounded to fp16 as the reference's separate ops round.  `highPrecision` (an fp32 down
+    projection) is not provided by the library."""
+
+    def __init__(self, count: int, configuration: LoRANetworkConfiguration, noBias: bool = False, flags: int = 0,
+                 name: str = ""):
+        if configuration.highPrecision:
+            raise NotImplementedError("LoRADense: highPrecision (fp32 down projection) is not available")
+        self.count, self.configuration, self.noBias, self.flags, self.name = count, configuration, noBias, flags, name
+        self.weight: Optional[QxTensor] = None
+        self.bias = None
+        self.down: Optional[QxTensor] = None  # [rank, in] fp16
+        self.up: Optional[QxTensor] = None    # [count, rank] fp16
+
+    def _padded(self):
+        """The pair with the rank padded by zero rows / columns to the tiled kernel's K granule (64): the zeros add
+        nothing, so the results are the same bit for bit, and the up projection avoids the slow any-shape kernel."""
+        key = (self.down.data.data_ptr(), self.up.data.data_ptr())
+        if getattr(self, "_pad_key", None) != key:
+            r = self.configuration.rank
+            rp = (r + 63) // 64 * 64
+            dn, up = self.down, self.up
+            if rp != r and self.down.qbits == 16 and self.up.qbits == 16:
+                torch = _torch()
+                d = torch.zeros((rp, dn.shape[1]), dtype=torch.float16, device=dn.data.device)
+                d[:r] = dn.data
+                u = torch.zeros((self.count, rp), dtype=torch.float16, device=up.data.device)
+                u[:, :r] = up.data
+                dn, up = QxTensor(d, 16, 0, tuple(d.shape)), QxTensor(u, 16, 0, tuple(u.shape))
+            self._pad_key, self._pad = key, (dn, up)
+        return self._pad
+
+    def __call__(self, x, post: Optional[DensePost] = None, stream=None):
+        if self.weight is None:
+            raise RuntimeError(f"LoRADense {self.name!r}: weight not loaded")
+        b = None if self.noBias else self.bias
+        if self.configuration.rank <= 0 or self.down is None or self.up is None:  # no matching LoRA keys: plain Dense
+            if post is None:
+                return dense_multi(x, [self.weight], [b], flags=self.flags, stream=stream)[0]
+            return dense_post(x, [self.weight], [b], [post], flags=self.flags, stream=stream)[0]
+        if self.down.shape[0] != self.configuration.rank or self.up.shape != (self.count, self.configuration.rank):
+            raise ValueError(f"LoRADense {self.name!r}: down / up shapes do not match rank and count")
+        dn, up = self._padded()
+        down = dense_post(x, [dn], [None], [DensePost(scale=self.configuration.scale)], stream=stream)[0]
+        branch = dense_multi(down, [up], [None], stream=stream)[0]
+        p = post or DensePost()
+        tail = DensePost(p.activation, p.gate, p.residual, p.keep_output, addend=branch.reshape(-1, self.count))
+        return dense_post(x, [self.weight], [b], [tail], flags=self.flags, stream=stream)[0]
 
 
 def _view4(t) -> _View4:

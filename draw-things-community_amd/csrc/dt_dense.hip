@@ -42,7 +42,11 @@ struct DenseWeight {
   const uint16_t* rot;
   int64_t rot_pos0;
   float eps;
-  // optional elementwise tail: activation, per-feature gate, accumulation into an fp32 residual stream
+  // optional elementwise tail: scalar scale, fp16 addend, activation, per-feature gate, accumulation into an
+  // fp32 residual stream
+  float scale;           // 1 = none
+  const uint16_t* add;   // [m, n] fp16 with row stride ld_add; null = none
+  int64_t ld_add;
   int32_t act;          // DT_ACT_*
   const uint16_t* gate;  // [n] or null
   float* res;            // [m, n] fp32 with row stride ld_res, updated in place; null = none
@@ -50,7 +54,8 @@ struct DenseWeight {
 };
 
 // The elementwise tail on one value that has already been rounded to fp16, with
-// the rounding the op-by-op graph applies: after the activation and after the gate.
+// the rounding the op-by-op graph applies: after the scale, after the addition,
+// after the activation and after the gate.
 __device__ __forceinline__ float act_gelu_tanh(float x) {
   const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
   const float e = __builtin_amdgcn_exp2f(u * 2.885390081777927f);  // exp(2u)
@@ -60,7 +65,10 @@ __device__ __forceinline__ float act_gelu_tanh(float x) {
 __device__ __forceinline__ float act_swish(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
 }
-__device__ __forceinline__ float post_value(float v, int act, bool has_gate, float gate) {
+__device__ __forceinline__ float post_value(float v, float scale, bool has_add, float add, int act, bool has_gate,
+                                            float gate) {
+  if (scale != 1.0f) v = (float)(half_t)(v * scale);
+  if (has_add) v = (float)(half_t)(v + add);
   if (act == DT_ACT_GELU_TANH) v = (float)(half_t)act_gelu_tanh(v);
   else if (act == DT_ACT_SWISH) v = (float)(half_t)act_swish(v);
   if (has_gate) v = (float)(half_t)(v * gate);
@@ -580,7 +588,9 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       const int64_t gmc = gm < g.m ? gm : 0;
       uint16_t* yrow = w.y ? w.y + gmc * w.ldy : nullptr;
       float* rrow = w.res ? w.res + gmc * w.ld_res : nullptr;
-      const bool vec = (!w.gate || (reinterpret_cast<uintptr_t>(w.gate) & 7) == 0) &&
+      const uint16_t* arow = w.add ? w.add + gmc * w.ld_add : nullptr;
+      const bool vec = (!w.add || (((w.ld_add & 3) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 7) == 0)) &&
+                       (!w.gate || (reinterpret_cast<uintptr_t>(w.gate) & 7) == 0) &&
                        (!w.bias || (reinterpret_cast<uintptr_t>(w.bias) & 7) == 0) &&
                        (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0)) &&
                        (!w.y || (((w.ldy & 3) == 0) && (reinterpret_cast<uintptr_t>(w.y) & 7) == 0));
@@ -590,6 +600,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         for (int gq = 0; gq < 4; gq++) {
           const int nn = n0 + wn * WN + i * 32 + 8 * gq + 4 * hi;
           float bq[4] = {0.f, 0.f, 0.f, 0.f}, gt[4] = {1.f, 1.f, 1.f, 1.f}, rr[4] = {0.f, 0.f, 0.f, 0.f}, pv[4];
+          float ad[4] = {0.f, 0.f, 0.f, 0.f};
           const bool full = vec && nn + 3 < w.n;
           if (gm < g.m) {
             if (full) {
@@ -603,6 +614,11 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
                 gt[0] = (float)bits_to_half((uint16_t)t2[0]); gt[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
                 gt[2] = (float)bits_to_half((uint16_t)t2[1]); gt[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
               }
+              if (arow) {
+                const uint2_t t2 = *reinterpret_cast<const uint2_t*>(arow + nn);
+                ad[0] = (float)bits_to_half((uint16_t)t2[0]); ad[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
+                ad[2] = (float)bits_to_half((uint16_t)t2[1]); ad[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
+              }
               if (rrow) {
                 const float4_t t4 = *reinterpret_cast<const float4_t*>(rrow + nn);
                 rr[0] = t4[0]; rr[1] = t4[1]; rr[2] = t4[2]; rr[3] = t4[3];
@@ -614,12 +630,13 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
                   if (w.bias) bq[e] = (float)bits_to_half(w.bias[nn + e]);
                   if (w.gate) gt[e] = (float)bits_to_half(w.gate[nn + e]);
                   if (rrow) rr[e] = rrow[nn + e];
+                  if (arow) ad[e] = (float)bits_to_half(arow[nn + e]);
                 }
             }
 #pragma unroll
             for (int e = 0; e < 4; e++) {
               const float v0 = (float)(half_t)(acc[i][j][4 * gq + e] + bq[e]);
-              pv[e] = post_value(v0, w.act, w.gate != nullptr, gt[e]);
+              pv[e] = post_value(v0, w.scale, arow != nullptr, ad[e], w.act, w.gate != nullptr, gt[e]);
               rr[e] += pv[e];
             }
             if (full) {
@@ -796,7 +813,8 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
 __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* __restrict__ x, int64_t ldx, int64_t m,
                                                              int64_t n, int64_t k, const uint8_t* __restrict__ wdata,
                                                              int qbits, int nib, const uint16_t* __restrict__ bias,
-                                                             uint16_t* __restrict__ y, int64_t ldy, int act,
+                                                             uint16_t* y, int64_t ldy, float scale,
+                                                             const uint16_t* add, int64_t ld_add, int act,
                                                              const uint16_t* __restrict__ gate, float* __restrict__ res,
                                                              int64_t ld_res) {
   int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -820,7 +838,8 @@ __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* _
   }
   if (bias) acc += (float)bits_to_half(bias[ni]);
   float v = (float)(half_t)acc;
-  v = post_value(v, act, gate != nullptr, gate ? (float)bits_to_half(gate[ni]) : 1.0f);
+  v = post_value(v, scale, add != nullptr, add ? (float)bits_to_half(add[mi * ld_add + ni]) : 0.f, act, gate != nullptr,
+                 gate ? (float)bits_to_half(gate[ni]) : 1.0f);
   if (res) res[mi * ld_res + ni] += v;
   if (y) y[mi * ldy + ni] = half_to_bits((half_t)v);
 }
@@ -863,7 +882,7 @@ static dt_status launch_tiled_qp(hipStream_t s, const DenseArgs& a, int qbits, i
 template <int BM, int BN>
 static dt_status launch_tiled_q(hipStream_t s, const DenseArgs& a, int qbits, int mode) {
   bool post = false;
-  for (int i = 0; i < kMaxWeights; i++) post = post || a.w[i].act != DT_ACT_NONE || a.w[i].gate || a.w[i].res;
+  for (int i = 0; i < kMaxWeights; i++) post = post || a.w[i].act != DT_ACT_NONE || a.w[i].gate || a.w[i].res || a.w[i].add || a.w[i].scale != 1.0f;
   return post ? launch_tiled_qp<BM, BN, true>(s, a, qbits, mode) : launch_tiled_qp<BM, BN, false>(s, a, qbits, mode);
 }
 
@@ -932,6 +951,9 @@ static dt_status validate_group(const HostGroup& h) {
       if (p.activation < DT_ACT_NONE || p.activation > DT_ACT_SWISH) return DT_INVALID;
       if (p.residual && ((reinterpret_cast<uintptr_t>(p.residual) & 3) || (h.W && h.K > 0 && p.ld_residual < h.W[i].count / h.K)))
         return DT_INVALID;
+      if (p.addend && ((reinterpret_cast<uintptr_t>(p.addend) & 1) || (h.W && h.K > 0 && p.ld_addend < h.W[i].count / h.K)))
+        return DT_INVALID;
+      if (!(p.scale == p.scale) || p.scale - p.scale != 0.f) return DT_INVALID;  // NaN or infinite
     }
   if (h.M > 0x7fffffff || h.K > 0x7fffffff) return DT_INVALID;
   for (int i = 0; i < h.n_weights; i++) {
@@ -966,6 +988,11 @@ static dt_status epilogue_pass(hipStream_t s, const HostGroup& h, int wi) {
   return qk_prep_launch(s, p);
 }
 
+// dt_dense_post::scale as the kernels take it: 0 (a zeroed struct) means none.
+static float post_scale(const HostGroup& h, int wi) {
+  return h.post && h.post[wi].scale != 0.f ? h.post[wi].scale : 1.0f;
+}
+
 // Appends weight wi of h to the launch; returns its number of N-tiles.
 static int add_weight(DenseArgs& a, int slot, const HostGroup& h, int wi, int tile_begin, int BN, bool fuse) {
   const int64_t n_rows = h.W[wi].count / h.K;
@@ -980,6 +1007,9 @@ static int add_weight(DenseArgs& a, int slot, const HostGroup& h, int wi, int ti
   d.rot = fuse ? h.epi[wi].rot : nullptr;
   d.rot_pos0 = fuse ? h.epi[wi].rot_pos0 : 0;
   d.eps = fuse ? h.epi[wi].eps : 0.f;
+  d.scale = post_scale(h, wi);
+  d.add = h.post ? h.post[wi].addend : nullptr;
+  d.ld_add = h.post ? h.post[wi].ld_addend : 0;
   d.act = h.post ? h.post[wi].activation : DT_ACT_NONE;
   d.gate = h.post ? h.post[wi].gate : nullptr;
   d.res = h.post ? h.post[wi].residual : nullptr;
@@ -1012,7 +1042,9 @@ static dt_status run_group(hipStream_t s, const HostGroup& h) {
         if ((outs + 255) / 256 > 0x7fffffff) return DT_NO_KERNEL;
         hipLaunchKernelGGL(dense_qx_generic_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, s, h.X, h.ldx,
                            M, n_rows0, K, static_cast<const uint8_t*>(w0.data), w0.qbits, w0.nib,
-                           h.bias ? h.bias[i] : nullptr, h.Y[i], h.ldy[i], h.post ? h.post[i].activation : DT_ACT_NONE,
+                           h.bias ? h.bias[i] : nullptr, h.Y[i], h.ldy[i], post_scale(h, i),
+                           h.post ? h.post[i].addend : nullptr, h.post ? h.post[i].ld_addend : 0,
+                           h.post ? h.post[i].activation : DT_ACT_NONE,
                            h.post ? h.post[i].gate : nullptr, h.post ? h.post[i].residual : nullptr,
                            h.post ? h.post[i].ld_residual : 0);
         dt_status st = launch_status();

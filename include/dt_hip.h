@@ -153,6 +153,9 @@ dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K, const ui
  * Dense followed by the elementwise tail of the feed-forward and residual paths
  * of a transformer block, applied in the GEMM epilogue in this order, each step
  * rounding to fp16 as the separate ops do:
+ *   scale      : scalar multiplier of the result; 0 or 1 = none (configuration.scale * downX, Models/LoRA.swift:129-134)
+ *   addend     : fp16 [M, N_i] with row stride ld_addend, added to the result: the low-rank branch of a
+ *                LoRADense, out = dense(x) + up(down(x)) (Models/LoRA.swift:117-140); may be Y[i] itself (in place)
  *   activation : DT_ACT_GELU_TANH  linear1(x).GELU(approximate: .tanh)  (Models/Flux1.swift:133-135, Models/Wan.swift:52-53)
  *                DT_ACT_SWISH      fc0(x).swish()                       (Models/Flux1.swift:122-123)
  *   gate       : [N_i] fp16, multiplies every output row ((xOut .* xChunks[2]), Models/Flux1.swift:246-250)
@@ -171,6 +174,9 @@ typedef struct {
   const uint16_t* gate;
   float* residual;
   int64_t ld_residual;
+  float scale;
+  const uint16_t* addend;
+  int64_t ld_addend;
 } dt_dense_post;
 
 dt_status dt_dense_qx_post_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,

@@ -358,6 +358,21 @@ def np_swish16(y16: np.ndarray) -> np.ndarray:
     return (x / (np.float32(1) + np.exp(-x))).astype(np.float16)
 
 
+def np_lora_branch16(X16: np.ndarray, down16: np.ndarray, up16: np.ndarray, scale: float = 1.0) -> np.ndarray:
+    """up(scale * down(x)) of a LoRADense, each op rounding to fp16 (Models/LoRA.swift:117-140): down [rank, in],
+    up [count, rank], both without bias; the scalar multiply is its own op and only exists when scale != 1."""
+    d = np_dense64(X16, down16).astype(np.float16)
+    if scale != 1:
+        d = (d.astype(np.float32) * np.float32(scale)).astype(np.float16)
+    return np_dense64(d, up16).astype(np.float16)
+
+
+def np_add16(a16: np.ndarray, b16: np.ndarray) -> np.ndarray:
+    """fp16 elementwise sum (out = dense(x) + up(...), Models/LoRA.swift:128-140); the float32 sum of two fp16 values
+    is exact, so one rounding."""
+    return (a16.astype(np.float32) + b16.astype(np.float32)).astype(np.float16)
+
+
 def np_gated_residual(res32: np.ndarray, y16: np.ndarray, gate16=None) -> np.ndarray:
     """res + float32(fp16(y * gate)); gate broadcast over rows."""
     y = y16 if gate16 is None else (y16.astype(np.float32) * gate16.astype(np.float32)[None, :]).astype(np.float16)

@@ -360,6 +360,73 @@ def test_dense_post_feed_forward_and_residual(dthip, oracle, torch_cuda, M, N, K
     assert float(big[:, :4].abs().max()) == 0 and float(big[:, 4 + N:].abs().max()) == 0
 
 
+@pytest.mark.parametrize("M,N,K,q,nib,rank,scale", [
+    (300, 512, 256, 6, 4096, 16, 1.0),     # rank below a K-tile: the up projection takes the generic kernel
+    (1100, 384, 128, 4, 512, 64, 0.5),     # tiled up projection, scaled branch
+    (513, 256, 192, 16, 0, 128, 0.75),     # plain fp16 base
+    (70, 100, 96, 6, 64, 8, 2.0),          # everything through the generic kernel
+])
+def test_lora_dense(dthip, oracle, torch_cuda, M, N, K, q, nib, rank, scale):
+    """LoRADense: dense(x) + up(scale * down(x)) with the base left palettized (Models/LoRA.swift:85-142).  The
+    epilogue's scale and addend steps are checked bit for bit on the device's own intermediates (exact op-by-op
+    rounding), the whole chain against the oracle's composition within the Dense bar."""
+    torch = torch_cuda
+    rng = np.random.default_rng(M + rank)
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    if q == 16:
+        Wh = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+        w, ref = dthip.QxTensor.from_f16(Wh), lambda b: oracle.C.dense(X, Wh, b)
+    else:
+        w, p = make_weight(dthip, oracle, rng, N, K, q, nib, std=0.05)
+        ref = lambda b: oracle.C.dense_qx(X, p, q, nib, N, b)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float16)
+    down = (rng.standard_normal((rank, K)) * 0.1).astype(np.float16)
+    up = (rng.standard_normal((N, rank)) * 0.1).astype(np.float16)
+    xd, bd = to_dev(torch, X), to_dev(torch, bias)
+    print("lora dense", M, N, K, q, rank, scale, flush=True)
+    layer = dthip.LoRADense(N, dthip.LoRANetworkConfiguration(rank, scale))
+    layer.weight, layer.bias = w, bd
+    layer.down, layer.up = dthip.QxTensor.from_f16(down), dthip.QxTensor.from_f16(up)
+    out = layer(xd).cpu().numpy()
+    # whole chain against the oracle
+    want = oracle.np_add16(ref(bias), oracle.np_lora_branch16(X, down, up, scale))
+    mx, rr = oracle.err_stats(out, want)
+    assert mx <= MAX_ABS and rr <= 2 * REL_RMS
+    # the steps one by one on the device's own intermediates: exact
+    # (the layer pads the rank to a multiple of 64 with zeros; the same padded pair is used here)
+    base = dthip.dense_multi(xd, [w], [bd])[0]
+    dn, upp = layer._padded()
+    assert dn.shape[0] % 64 == 0 and upp.shape == (N, dn.shape[0])
+    d0 = dthip.dense_multi(xd, [dn], [None])[0]
+    d1 = dthip.dense_post(xd, [dn], [None], [dthip.DensePost(scale=scale)])[0]
+    assert np.array_equal(d1.cpu().numpy().view(np.uint16),
+                          (d0.cpu().numpy().astype(np.float32) * np.float32(scale)).astype(np.float16).view(np.uint16))
+    assert float(d1[:, rank:].abs().max()) == 0 if dn.shape[0] > rank else True
+    branch = dthip.dense_multi(d1, [upp], [None])[0]
+    assert np.array_equal(out.view(np.uint16), oracle.np_add16(base.cpu().numpy(), branch.cpu().numpy()).view(np.uint16))
+    # the unpadded pair (any-shape kernel where the rank is no multiple of 64) agrees within the Dense bar
+    b2 = dthip.dense_multi(dthip.dense_post(xd, [layer.down], [None], [dthip.DensePost(scale=scale)])[0], [layer.up], [None])[0]
+    mx, rr = oracle.err_stats(b2.cpu().numpy(), branch.cpu().numpy())
+    assert mx <= MAX_ABS and rr <= 2 * REL_RMS
+    # in place: the branch buffer receives the sum; a row-strided addend view; then GELU behind the sum
+    buf = branch.clone()
+    o = dthip.dense_post(xd, [w], [bd], [dthip.DensePost(addend=buf)], outs=[buf])[0]
+    assert np.array_equal(o.cpu().numpy().view(np.uint16), out.view(np.uint16))
+    wide = torch.zeros((M, N + 8), dtype=torch.float16, device="cuda")
+    wide[:, 4:4 + N].copy_(branch)
+    o = dthip.dense_post(xd, [w], [bd], [dthip.DensePost(dthip.ACT_GELU_TANH, addend=wide[:, 4:4 + N])])[0]
+    g = layer(xd, post=dthip.DensePost(dthip.ACT_GELU_TANH))
+    assert torch.equal(o, g)
+    # one fp16 ulp, or 2^-19 where GELU's 1 + tanh cancels (inputs below -3: results of 1e-4 and less)
+    got16, want16 = o.cpu().numpy(), oracle.np_gelu_tanh16(out)
+    tol = np.maximum(np.spacing(np.abs(want16)).astype(np.float32), np.float32(2.0 ** -19))
+    assert np.all(np.abs(got16.astype(np.float32) - want16.astype(np.float32)) <= tol)
+    # rank 0 / no matching keys: the plain Dense
+    plain = dthip.LoRADense(N, dthip.LoRANetworkConfiguration(0))
+    plain.weight, plain.bias = w, bd
+    assert torch.equal(plain(xd), base)
+
+
 def test_dense_post_bad_args(dthip, oracle, torch_cuda):
     torch = torch_cuda
     rng = np.random.default_rng(9)
@@ -371,6 +438,12 @@ def test_dense_post_bad_args(dthip, oracle, torch_cuda):
         dthip.dense_post(x, [w], [None], [dthip.DensePost(residual=torch.zeros((4, 64), dtype=torch.float16, device="cuda"))])
     with pytest.raises(ValueError):
         dthip.dense_post(x, [w], [None], [dthip.DensePost(gate=torch.zeros(3, dtype=torch.float16, device="cuda"))])
+    with pytest.raises(ValueError):
+        dthip.dense_post(x, [w], [None], [dthip.DensePost(addend=torch.zeros((4, 32), dtype=torch.float16, device="cuda"))])
+    with pytest.raises(dthip.DtError):
+        dthip.dense_post(x, [w], [None], [dthip.DensePost(scale=float("inf"))])
+    with pytest.raises(NotImplementedError):
+        dthip.LoRADense(64, dthip.LoRANetworkConfiguration(4, highPrecision=True))
 
 
 def test_dense_wan_full_size_sampled(dthip, oracle, torch_cuda):

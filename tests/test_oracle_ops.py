@@ -276,3 +276,40 @@ def test_elementwise_tails_pinned(oracle):
     g2 = np.array([1.0009765625], np.float16)
     # (1 + 2^-10)^2 = 1 + 2^-9 + 2^-20 rounds to 1 + 2^-9 in fp16 before it reaches the fp32 stream
     assert oracle.np_gated_residual(np.zeros((1, 1), np.float32), y2, g2)[0, 0] == np.float32(1 + 2.0 ** -9)
+
+
+def test_lora_branch_pinned(oracle):
+    """The low-rank branch up(scale * down(x)) and the fp16 sum, against what the mathematics fixes: exact small
+    integers, the rank-1 outer-product form, exact doubling by a power-of-two scale, the merged-weight form
+    x (up down)^T within fp16 rounding, and where the intermediate rounding must show."""
+    rng = np.random.default_rng(5)
+    # small integers: every product and sum is exact in fp16
+    X = rng.integers(-3, 4, (7, 8)).astype(np.float16)
+    D = rng.integers(-2, 3, (4, 8)).astype(np.float16)
+    U = rng.integers(-2, 3, (6, 4)).astype(np.float16)
+    want = (X.astype(np.int64) @ D.astype(np.int64).T) @ U.astype(np.int64).T
+    assert np.array_equal(oracle.np_lora_branch16(X, D, U).astype(np.int64), want)
+    assert np.array_equal(oracle.np_lora_branch16(X, D, U, 2.0).astype(np.int64), 2 * want)
+    # a transposed operand or a swapped pair fails the shapes or the values
+    assert oracle.np_lora_branch16(X, D, U).shape == (7, 6)
+    # rank 1: branch[m, n] = u[n] * fp16(v . x[m])
+    v = rng.standard_normal((1, 8)).astype(np.float16)
+    u = rng.standard_normal((6, 1)).astype(np.float16)
+    Xr = rng.standard_normal((5, 8)).astype(np.float16)
+    d = (Xr.astype(np.float64) @ v.astype(np.float64).T).astype(np.float16)
+    assert np.array_equal(oracle.np_lora_branch16(Xr, v, u), (d.astype(np.float64) * u.astype(np.float64).T).astype(np.float16))
+    # merged weight: equal up to the fp16 rounding of the intermediate and the output
+    Dg = (rng.standard_normal((16, 64)) * 0.1).astype(np.float16)
+    Ug = (rng.standard_normal((32, 16)) * 0.1).astype(np.float16)
+    Xg = rng.standard_normal((9, 64)).astype(np.float16)
+    merged = Xg.astype(np.float64) @ (Ug.astype(np.float64) @ Dg.astype(np.float64)).T
+    got = oracle.np_lora_branch16(Xg, Dg, Ug, 0.5).astype(np.float64)
+    assert np.max(np.abs(got - 0.5 * merged)) <= 4e-3 * np.abs(merged).max()
+    # scale by 1/3 is its own rounding step: not the same as scaling the output
+    third = oracle.np_lora_branch16(Xg, Dg, Ug, 1 / 3)
+    assert np.max(np.abs(third.astype(np.float64) - merged / 3)) <= 4e-3 * np.abs(merged).max()
+    # fp16 sum: exact where representable, one rounding (ties to even) where not
+    a = np.array([1.0, 2048.0, 2048.0, -0.5], np.float16)
+    b = np.array([0.5, 1.0, 3.0, 0.5], np.float16)
+    assert np.array_equal(oracle.np_add16(a, b), np.array([1.5, 2048.0, 2052.0, 0.0], np.float16))
+
