@@ -35,6 +35,7 @@ ABI_SYMBOLS = (
     "dt_dense_qx_grouped_f16",
     "dt_dense_qx_post_f16",
     "dt_qk_norm_rope_f16",
+    "dt_layernorm_modulate_f16",
     "dt_sdpa_f16",
     "dt_sdpa_workspace_bytes",
 )
@@ -124,6 +125,8 @@ def lib():
         L.dt_dense_qx_grouped_f16.restype = i32
         L.dt_dense_qx_grouped_f16.argtypes = [vp, i32, ctypes.POINTER(_DenseGroup), ctypes.c_uint32]
         L.dt_qk_norm_rope_f16.argtypes = [vp, _View4, i32, i64, i32, i32, vp, f32, i32, vp, i64, f32]
+        L.dt_layernorm_modulate_f16.restype = i32
+        L.dt_layernorm_modulate_f16.argtypes = [vp, i64, i64, vp, i64, vp, vp, i32, f32, vp, i64]
         L.dt_sdpa_f16.restype = i32
         L.dt_sdpa_f16.argtypes = [vp, i32, i32, i32, i32, i32, ctypes.POINTER(_Segment), i32,
                                   ctypes.POINTER(_Segment), ctypes.POINTER(_Segment), vp, vp, f32, _View4, f32,
@@ -540,6 +543,56 @@ class RMSNorm:
             qk_norm_rope_(_as_heads(y), self.weight, self.epsilon, False, stream=stream)
             return y
         raise DtError("RMSNorm", DT_NO_KERNEL)
+
+
+MOD_F16, MOD_F32 = 0, 1
+
+
+def layernorm_modulate(x, scale=None, shift=None, epsilon: float = 1e-6, out=None, stream=None):
+    """LayerNorm(epsilon:, axis: [last], elementwiseAffine: false) of the fp32 stream `x` [..., C], then the adaLN
+    modulation, fp16 out.  fp16 `scale` / `shift` [C]: `norm(x).to(.Float16) .* scale + shift` (Models/Flux1.swift:
+    172-173); fp32 ones: `(norm(x) .* (scale + 1) + shift).to(.Float16)` (Models/Wan.swift:217-221)."""
+    torch = _torch()
+    if not (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.float32):
+        raise TypeError("x must be a float32 CUDA tensor")
+    C = x.shape[-1]
+    x2 = x.reshape(-1, C)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    mods = [t for t in (scale, shift) if t is not None]
+    dtypes = {t.dtype for t in mods}
+    if len(dtypes) > 1 or not dtypes <= {torch.float16, torch.float32}:
+        raise TypeError("scale and shift must both be float16 or both be float32")
+    for t in mods:
+        if not t.is_cuda or t.numel() != C or not t.is_contiguous():
+            raise ValueError("scale / shift must be contiguous CUDA vectors of C elements")
+    mod = MOD_F32 if dtypes == {torch.float32} else MOD_F16
+    if out is None:
+        out = torch.empty((M, C), dtype=torch.float16, device=x.device)
+    elif out.dtype != torch.float16 or out.shape != (M, C) or out.stride(1) != 1:
+        raise ValueError("out must be an [M, C] float16 view with contiguous rows")
+    st = lib().dt_layernorm_modulate_f16(_stream_ptr(stream), M, C, x2.data_ptr(), x2.stride(0),
+                                         None if scale is None else scale.data_ptr(),
+                                         None if shift is None else shift.data_ptr(), mod, float(epsilon),
+                                         out.data_ptr(), out.stride(0))
+    _check("dt_layernorm_modulate_f16", st)
+    return out.reshape(tuple(x.shape[:-1]) + (C,)) if out.is_contiguous() else out
+
+
+class LayerNorm:
+    """LayerNorm(epsilon:axis:elementwiseAffine: false) on the last axis of an fp32 tensor, result cast to fp16
+    (`xNorm1(x).to(.Float16)`, Models/Flux1.swift:172-173).  The affine form is not on the accelerated path."""
+
+    def __init__(self, epsilon: float, axis: Sequence[int], elementwiseAffine: bool = True, name: str = ""):
+        if elementwiseAffine:
+            raise NotImplementedError("LayerNorm with elementwiseAffine is not provided")
+        self.epsilon, self.axis, self.name = epsilon, list(axis), name
+
+    def __call__(self, x, stream=None):
+        if self.axis != [x.dim() - 1]:
+            raise ValueError("LayerNorm: only the last axis is supported")
+        return layernorm_modulate(x, None, None, self.epsilon, stream=stream)
 
 
 def _as_heads(y):

@@ -1,0 +1,174 @@
+// K4: LayerNorm(elementwiseAffine: false) over the last axis of an fp32 residual
+// stream followed by the adaLN modulation, fp16 out -- the op in front of every
+// Dense of a DiT block.  HBM-bound: 4 bytes read and 2 written per element.
+// One wave per row; the row stays in registers between the mean, the variance
+// and the output pass, so memory is touched once.
+#include "dt_common.h"
+
+namespace dt {
+
+__device__ __forceinline__ float wave_sum64(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+__device__ __forceinline__ float round16(float v) { return (float)(half_t)v; }
+
+// One normalised value through the modulation (sc, sh already widened to float).
+//   DT_MOD_F16: fp16(fp16(fp16(n) * scale) + shift), scale and shift fp16
+//   DT_MOD_F32: fp16(n * (scale + 1) + shift), scale and shift fp32
+template <int MOD>
+__device__ __forceinline__ uint16_t modulate(float n, bool has_scale, float sc, bool has_shift, float sh) {
+  if constexpr (MOD == DT_MOD_F16) {
+    n = round16(n);
+    if (has_scale) n = round16(n * sc);
+    if (has_shift) n = round16(n + sh);
+  } else {
+    if (has_scale) n = n * (sc + 1.0f);
+    if (has_shift) n = n + sh;
+  }
+  return half_to_bits((half_t)n);
+}
+
+template <int MOD>
+__device__ __forceinline__ float mod_at(const void* p, int64_t c) {
+  if constexpr (MOD == DT_MOD_F16) return (float)bits_to_half(static_cast<const uint16_t*>(p)[c]);
+  else return static_cast<const float*>(p)[c];
+}
+// four consecutive values starting at element c (c % 4 == 0, vector aligned)
+template <int MOD>
+__device__ __forceinline__ void mod_at4(const void* p, int c, float (&o)[4]) {
+  if constexpr (MOD == DT_MOD_F16) {
+    const uint2_t t = *reinterpret_cast<const uint2_t*>(static_cast<const uint16_t*>(p) + c);
+    o[0] = (float)bits_to_half((uint16_t)t[0]); o[1] = (float)bits_to_half((uint16_t)(t[0] >> 16));
+    o[2] = (float)bits_to_half((uint16_t)t[1]); o[3] = (float)bits_to_half((uint16_t)(t[1] >> 16));
+  } else {
+    const float4_t t = *reinterpret_cast<const float4_t*>(static_cast<const float*>(p) + c);
+    o[0] = t[0]; o[1] = t[1]; o[2] = t[2]; o[3] = t[3];
+  }
+}
+
+struct AdaLnArgs {
+  const float* x;
+  int64_t ldx;
+  int64_t m, c;
+  const void* scale;
+  const void* shift;
+  float eps;
+  uint16_t* y;
+  int64_t ldy;
+};
+
+// Rows of up to NV * 256 elements, C % 4 == 0, 16-byte aligned rows: lane l
+// holds the float4 at element 256 i + 4 l of every 256-element chunk i.
+template <int NV, int MOD>
+__global__ void __launch_bounds__(256) adaln_rows_kernel(const AdaLnArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.m) return;
+  const float* xr = a.x + row * a.ldx;
+  uint16_t* yr = a.y + row * a.ldy;
+  const int c = (int)a.c;
+  float4_t v[NV];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int e = i * 256 + lane * 4;
+    v[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    if (e < c) v[i] = *reinterpret_cast<const float4_t*>(xr + e);
+    s += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
+  }
+  const float mean = wave_sum64(s) / (float)c;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int e = i * 256 + lane * 4;
+    if (e < c) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        v[i][j] -= mean;
+        q += v[i][j] * v[i][j];
+      }
+    }
+  }
+  const float inv = 1.0f / sqrtf(wave_sum64(q) / (float)c + a.eps);
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int e = i * 256 + lane * 4;
+    if (e < c) {
+      uint16_t o[4];
+      float sc[4] = {0.f, 0.f, 0.f, 0.f}, sh[4] = {0.f, 0.f, 0.f, 0.f};
+      if (a.scale) mod_at4<MOD>(a.scale, e, sc);
+      if (a.shift) mod_at4<MOD>(a.shift, e, sh);
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        o[j] = modulate<MOD>(v[i][j] * inv, a.scale != nullptr, sc[j], a.shift != nullptr, sh[j]);
+      *reinterpret_cast<uint2_t*>(yr + e) =
+          uint2_t{(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
+    }
+  }
+}
+
+// Any width and alignment: three passes over the row (it stays in cache), scalar accesses.
+template <int MOD>
+__global__ void __launch_bounds__(256) adaln_generic_kernel(const AdaLnArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.m) return;
+  const float* xr = a.x + row * a.ldx;
+  uint16_t* yr = a.y + row * a.ldy;
+  float s = 0.f;
+  for (int64_t e = lane; e < a.c; e += 64) s += xr[e];
+  const float mean = wave_sum64(s) / (float)a.c;
+  float q = 0.f;
+  for (int64_t e = lane; e < a.c; e += 64) {
+    const float d = xr[e] - mean;
+    q += d * d;
+  }
+  const float inv = 1.0f / sqrtf(wave_sum64(q) / (float)a.c + a.eps);
+  for (int64_t e = lane; e < a.c; e += 64)
+    yr[e] = modulate<MOD>((xr[e] - mean) * inv, a.scale != nullptr, a.scale ? mod_at<MOD>(a.scale, e) : 0.f,
+                          a.shift != nullptr, a.shift ? mod_at<MOD>(a.shift, e) : 0.f);
+}
+
+template <int MOD>
+static void launch_adaln(hipStream_t s, const AdaLnArgs& a, bool vec) {
+  const dim3 grid((unsigned)((a.m + 3) / 4)), block(256);
+  if (!vec || a.c > 32 * 256) {
+    hipLaunchKernelGGL((adaln_generic_kernel<MOD>), grid, block, 0, s, a);
+    return;
+  }
+  const int nv = (int)((a.c + 255) / 256);
+  if (nv <= 4) hipLaunchKernelGGL((adaln_rows_kernel<4, MOD>), grid, block, 0, s, a);
+  else if (nv <= 8) hipLaunchKernelGGL((adaln_rows_kernel<8, MOD>), grid, block, 0, s, a);
+  else if (nv <= 12) hipLaunchKernelGGL((adaln_rows_kernel<12, MOD>), grid, block, 0, s, a);
+  else if (nv <= 16) hipLaunchKernelGGL((adaln_rows_kernel<16, MOD>), grid, block, 0, s, a);
+  else if (nv <= 20) hipLaunchKernelGGL((adaln_rows_kernel<20, MOD>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((adaln_rows_kernel<32, MOD>), grid, block, 0, s, a);
+}
+
+}  // namespace dt
+
+DT_EXPORT dt_status dt_layernorm_modulate_f16(dt_stream stream, int64_t M, int64_t C, const float* X, int64_t ldx,
+                                              const void* scale, const void* shift, int32_t mod, float eps,
+                                              uint16_t* Y, int64_t ldy) {
+  using namespace dt;
+  if (M < 0 || C <= 0 || (mod != DT_MOD_F16 && mod != DT_MOD_F32)) return DT_INVALID;
+  if (!(eps >= 0.f) || eps - eps != 0.f) return DT_INVALID;
+  if (M == 0) return DT_OK;
+  if (!X || !Y || ldx < C || ldy < C) return DT_INVALID;
+  if ((reinterpret_cast<uintptr_t>(X) & 3) || (reinterpret_cast<uintptr_t>(Y) & 1)) return DT_INVALID;
+  const uintptr_t vec_align = mod == DT_MOD_F16 ? 1 : 3;
+  if ((reinterpret_cast<uintptr_t>(scale) & vec_align) || (reinterpret_cast<uintptr_t>(shift) & vec_align)) return DT_INVALID;
+  if ((M + 3) / 4 > 0x7fffffff) return DT_NO_KERNEL;
+  if (!device_ok()) return DT_NO_KERNEL;
+  AdaLnArgs a{X, ldx, M, C, scale, shift, eps, Y, ldy};
+  const bool vec = (C % 4 == 0) && (ldx % 4 == 0) && (ldy % 4 == 0) && (reinterpret_cast<uintptr_t>(X) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(Y) & 7) == 0 &&
+                   (reinterpret_cast<uintptr_t>(scale) & (mod == DT_MOD_F16 ? 7 : 15)) == 0 &&
+                   (reinterpret_cast<uintptr_t>(shift) & (mod == DT_MOD_F16 ? 7 : 15)) == 0;
+  if (mod == DT_MOD_F16) launch_adaln<DT_MOD_F16>(as_stream(stream), a, vec);
+  else launch_adaln<DT_MOD_F32>(as_stream(stream), a, vec);
+  return launch_status();
+}

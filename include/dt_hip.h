@@ -185,6 +185,27 @@ dt_status dt_dense_qx_post_f16(dt_stream stream, int64_t M, int64_t K, const uin
                                uint32_t flags);
 
 /*
+ * LayerNorm(epsilon:, axis: [last], elementwiseAffine: false) of the fp32
+ * residual stream followed by the adaLN modulation and the cast to fp16: the
+ * op in front of the attention and feed-forward Dense layers of a DiT block.
+ *   DT_MOD_F16 : y = fp16(fp16(fp16(norm(x)) * scale) + shift), scale / shift fp16 [C]
+ *                (xNorm1(x).to(.Float16) .* xChunks[1] + xChunks[0], Models/Flux1.swift:172-173, 281-282)
+ *   DT_MOD_F32 : y = fp16(norm(x) * (scale + 1) + shift), scale / shift fp32 [C]
+ *                ((xNorm2(out) .* (chunks[4] + 1) + chunks[3]).to(.Float16), Models/Wan.swift:217-221)
+ * norm(x) = (x - mean) / sqrt(var + eps) with the biased variance, in fp32.
+ * X: [M, C] fp32 with row stride ldx; Y: [M, C] fp16 with row stride ldy; scale
+ * and shift are broadcast over rows and may be NULL.  Rows that are 16-byte
+ * aligned with C % 4 == 0 and C <= 8192 stay in registers (one read, one write);
+ * anything else takes a three-pass kernel with the same results.
+ */
+#define DT_MOD_F16 0
+#define DT_MOD_F32 1
+
+dt_status dt_layernorm_modulate_f16(dt_stream stream, int64_t M, int64_t C, const float* X, int64_t ldx,
+                                    const void* scale, const void* shift, int32_t mod, float eps,
+                                    uint16_t* Y, int64_t ldy);
+
+/*
  * Several independent Dense problems (each an X with its weights, arguments as
  * for dt_dense_qx_heads_f16) enqueued together.  The context (text) and image
  * streams of a joint block apply different weights to different token sets

@@ -358,6 +358,30 @@ def np_swish16(y16: np.ndarray) -> np.ndarray:
     return (x / (np.float32(1) + np.exp(-x))).astype(np.float16)
 
 
+def np_layernorm_modulate16(x32: np.ndarray, scale=None, shift=None, eps: float = 1e-6, mod: str = "f16") -> np.ndarray:
+    """LayerNorm(epsilon:, axis: [last], elementwiseAffine: false) of an fp32 stream, then the adaLN modulation, fp16
+    out.  mod "f16": fp16(fp16(fp16(norm) * scale) + shift) with fp16 scale / shift -- xNorm1(x).to(.Float16) .*
+    xChunks[1] + xChunks[0] (Models/Flux1.swift:172-173, 281-282).  mod "f32": fp16(norm * (scale + 1) + shift) with
+    fp32 scale / shift -- (xNorm2(out) .* (chunks[4] + 1) + chunks[3]).to(.Float16) (Models/Wan.swift:217-221).
+    Statistics in float64 (biased variance), the normalised value rounded to float32 as the fp32 op leaves it."""
+    x = x32.astype(np.float64)
+    mean = x.mean(axis=-1, keepdims=True)
+    var = ((x - mean) ** 2).mean(axis=-1, keepdims=True)
+    n = ((x - mean) / np.sqrt(var + eps)).astype(np.float32)
+    if mod == "f16":
+        y = n.astype(np.float16)
+        if scale is not None:
+            y = (y.astype(np.float32) * scale.astype(np.float16).astype(np.float32)).astype(np.float16)
+        if shift is not None:
+            y = (y.astype(np.float32) + shift.astype(np.float16).astype(np.float32)).astype(np.float16)
+        return y
+    if scale is not None:
+        n = n * (scale.astype(np.float32) + np.float32(1))
+    if shift is not None:
+        n = n + shift.astype(np.float32)
+    return n.astype(np.float16)
+
+
 def np_lora_branch16(X16: np.ndarray, down16: np.ndarray, up16: np.ndarray, scale: float = 1.0) -> np.ndarray:
     """up(scale * down(x)) of a LoRADense, each op rounding to fp16 (Models/LoRA.swift:117-140): down [rank, in],
     up [count, rank], both without bias; the scalar multiply is its own op and only exists when scale != 1."""

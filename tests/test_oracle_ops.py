@@ -313,3 +313,46 @@ def test_lora_branch_pinned(oracle):
     b = np.array([0.5, 1.0, 3.0, 0.5], np.float16)
     assert np.array_equal(oracle.np_add16(a, b), np.array([1.5, 2048.0, 2052.0, 0.0], np.float16))
 
+
+
+def test_layernorm_modulate_pinned(oracle):
+    """LayerNorm + adaLN modulation against a library routine (torch layer_norm, fp32) and what the mathematics fixes:
+    zero mean / unit variance, invariance under a shift of the input, the two-valued row's closed form, the constant
+    row, and the place of each rounding."""
+    import torch
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((6, 96)) * 3 + 1.5).astype(np.float32)
+    plain = oracle.np_layernorm_modulate16(x, None, None, 1e-6, "f32").astype(np.float64)
+    ref = torch.nn.functional.layer_norm(torch.from_numpy(x), (96,), eps=1e-6).numpy().astype(np.float64)
+    assert np.max(np.abs(plain - ref)) <= 2.0 ** -10 * np.maximum(1, np.abs(ref)).max()
+    assert np.max(np.abs(plain.mean(axis=1))) < 2e-3 and np.max(np.abs(plain.var(axis=1) - 1)) < 5e-3
+    # LN(x + c) = LN(x): the mean is subtracted, not ignored
+    moved = oracle.np_layernorm_modulate16(x + np.float32(8), None, None, 1e-6, "f32").astype(np.float64)
+    assert np.max(np.abs(moved - plain)) <= 2.0 ** -9 * np.abs(plain).max()
+    # a row of +a / -a: mean 0, variance a^2 -> +-1 / sqrt(1 + eps / a^2); eps inside the root, added to the variance
+    a = np.float32(0.01)
+    row = np.tile(np.array([a, -a], np.float32), 8)[None, :]
+    want = 1 / np.sqrt(1 + 1e-2 / float(a) ** 2)
+    got = oracle.np_layernorm_modulate16(row, None, None, 1e-2, "f32").astype(np.float64)
+    assert np.allclose(got, np.tile([want, -want], 8)[None, :], rtol=2e-3)
+    # constant row -> zeros -> the shift alone
+    sh = rng.standard_normal(16).astype(np.float16)
+    const = np.full((1, 16), 3.25, np.float32)
+    assert np.array_equal(oracle.np_layernorm_modulate16(const, None, sh, 1e-6, "f16"), sh[None, :])
+    # the two modes: "f16" rounds three times and multiplies by scale; "f32" adds 1 to scale and rounds once
+    sc16 = (1 + 0.2 * rng.standard_normal(96)).astype(np.float16)
+    sh16 = rng.standard_normal(96).astype(np.float16)
+    n16 = ref.astype(np.float32).astype(np.float16)
+    step = (n16.astype(np.float32) * sc16.astype(np.float32)).astype(np.float16)
+    want16 = (step.astype(np.float32) + sh16.astype(np.float32)).astype(np.float16)
+    got16 = oracle.np_layernorm_modulate16(x, sc16, sh16, 1e-6, "f16")
+    assert np.max(np.abs(got16.astype(np.float64) - want16.astype(np.float64))) <= 2e-3 * np.maximum(1, np.abs(want16)).max()
+    sc32 = (0.2 * rng.standard_normal(96)).astype(np.float32)
+    sh32 = rng.standard_normal(96).astype(np.float32)
+    want32 = ref * (sc32.astype(np.float64) + 1) + sh32.astype(np.float64)
+    got32 = oracle.np_layernorm_modulate16(x, sc32, sh32, 1e-6, "f32").astype(np.float64)
+    assert np.max(np.abs(got32 - want32)) <= 2.0 ** -10 * np.maximum(1, np.abs(want32)).max()
+    # scale = 0 in "f32" mode leaves the normalised value (the +1), in "f16" mode it zeroes it
+    z32 = oracle.np_layernorm_modulate16(x, np.zeros(96, np.float32), None, 1e-6, "f32")
+    assert np.array_equal(z32, oracle.np_layernorm_modulate16(x, None, None, 1e-6, "f32"))
+    assert not oracle.np_layernorm_modulate16(x, np.zeros(96, np.float16), None, 1e-6, "f16").any()
