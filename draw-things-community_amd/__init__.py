@@ -70,7 +70,8 @@ class _DensePost(ctypes.Structure):
 class _DenseGroup(ctypes.Structure):
     _fields_ = [("M", ctypes.c_int64), ("K", ctypes.c_int64), ("X", ctypes.c_void_p), ("ldx", ctypes.c_int64),
                 ("W", ctypes.c_void_p), ("n_weights", ctypes.c_int32), ("bias", ctypes.c_void_p),
-                ("Y", ctypes.c_void_p), ("ldy", ctypes.c_void_p), ("epi", ctypes.c_void_p)]
+                ("Y", ctypes.c_void_p), ("ldy", ctypes.c_void_p), ("epi", ctypes.c_void_p),
+                ("post", ctypes.c_void_p)]
 
 
 class _Segment(ctypes.Structure):
@@ -367,13 +368,10 @@ class DensePost:
         self.scale, self.addend = scale, addend
 
 
-def dense_post(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]], posts: Sequence[Optional[DensePost]],
-               outs=None, flags: int = 0, stream=None):
-    """Dense ops sharing `x`, each followed by its DensePost tail inside the GEMM epilogue (the feed-forward's
-    linear1 -> GELU and the gated residual additions of a transformer block).  Returns the fp16 outputs (None where
-    a projection only accumulates into its residual)."""
+def _marshal_posts(posts, weights, M, Y, outs):
+    """dt_dense_post array for the DensePost tails of one problem; clears Y / outs entries that only accumulate."""
     torch = _torch()
-    x2, M, K, n, W, B, Y, LDY, _, outs = _marshal_dense(x, weights, biases, outs, None)
+    n = len(weights)
     P = (_DensePost * n)()
     for i, p in enumerate(posts):
         if p is None:
@@ -402,6 +400,16 @@ def dense_post(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]
                 raise ValueError("addend must be an [M, N] view with contiguous rows")
             ap, lda = a2.data_ptr(), a2.stride(0)
         P[i] = _DensePost(p.activation, None if p.gate is None else p.gate.data_ptr(), rp, ldr, float(p.scale), ap, lda)
+    return P
+
+
+def dense_post(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]], posts: Sequence[Optional[DensePost]],
+               outs=None, flags: int = 0, stream=None):
+    """Dense ops sharing `x`, each followed by its DensePost tail inside the GEMM epilogue (the feed-forward's
+    linear1 -> GELU and the gated residual additions of a transformer block).  Returns the fp16 outputs (None where
+    a projection only accumulates into its residual)."""
+    x2, M, K, n, W, B, Y, LDY, _, outs = _marshal_dense(x, weights, biases, outs, None)
+    P = _marshal_posts(posts, weights, M, Y, outs)
     st = lib().dt_dense_qx_post_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, P, flags)
     _check("dt_dense_qx_post_f16", st)
     lead = tuple(x.shape[:-1])
@@ -411,16 +419,22 @@ def dense_post(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]
 
 def dense_grouped(problems: Sequence[dict], flags: int = 0, stream=None):
     """Independent Dense problems enqueued together (the context and image projections of a joint block).  Each
-    problem is a dict with the arguments of dense_multi: x, weights, biases, and optionally outs, epilogues.
-    Returns one list of outputs per problem."""
+    problem is a dict with the arguments of dense_multi or dense_post: x, weights, biases, and optionally outs and
+    either epilogues or posts.  Returns one list of outputs per problem (None where a projection only accumulates
+    into its residual)."""
     keep = [_marshal_dense(p["x"], p["weights"], p["biases"], p.get("outs"), p.get("epilogues")) for p in problems]
     G = (_DenseGroup * len(keep))()
     cast = lambda a: None if a is None else ctypes.addressof(a)  # the arrays stay alive in `keep` until the call returns
+    posts = []
     for i, (x2, M, K, n, W, B, Y, LDY, E, outs) in enumerate(keep):
-        G[i] = _DenseGroup(M, K, x2.data_ptr(), x2.stride(0), cast(W), n, cast(B), cast(Y), cast(LDY), cast(E))
+        P = None
+        if problems[i].get("posts") is not None:
+            P = _marshal_posts(problems[i]["posts"], problems[i]["weights"], M, Y, outs)
+        posts.append(P)
+        G[i] = _DenseGroup(M, K, x2.data_ptr(), x2.stride(0), cast(W), n, cast(B), cast(Y), cast(LDY), cast(E), cast(P))
     st = lib().dt_dense_qx_grouped_f16(_stream_ptr(stream), len(keep), G, flags)
     _check("dt_dense_qx_grouped_f16", st)
-    return [_shape_outs(p["x"], k[1], k[9]) for p, k in zip(problems, keep)]
+    return [[None if o is None else _shape_outs(p["x"], k[1], [o])[0] for o in k[9]] for p, k in zip(problems, keep)]
 
 
 class Dense:

@@ -1120,6 +1120,13 @@ static bool run_groups_fused(hipStream_t s, const HostGroup* hs, int n, dt_statu
     total_w += h.n_weights;
   }
   if (!big || total_w > kMaxWeights) return false;
+  // the kernel variant with the elementwise tail has no fused head epilogue: such problems do not share a launch
+  bool any_post = false, any_epi = false;
+  for (int gi = 0; gi < n; gi++) {
+    any_post = any_post || hs[gi].post != nullptr;
+    for (int i = 0; i < hs[gi].n_weights; i++) any_epi = any_epi || hs[gi].wants_epi(i);
+  }
+  if (any_post && any_epi) return false;
   constexpr int BM = 256, BN = 256;
   DenseArgs a;
   int cnt = 0;
@@ -1198,7 +1205,7 @@ DT_EXPORT dt_status dt_dense_qx_grouped_f16(dt_stream stream, int32_t n_groups, 
   int n = 0;
   for (int i = 0; i < n_groups; i++) {
     const dt_dense_group& d = groups[i];
-    const HostGroup h{d.M, d.K, d.X, d.ldx, d.W, d.n_weights, d.bias, d.Y, d.ldy, d.epi, nullptr};
+    const HostGroup h{d.M, d.K, d.X, d.ldx, d.W, d.n_weights, d.bias, d.Y, d.ldy, d.epi, d.post};
     dt_status st = validate_group(h);
     if (st != DT_OK) return st;
     if (h.M > 0) hs[n++] = h;

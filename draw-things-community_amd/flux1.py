@@ -1,0 +1,97 @@
+"""Flux.1 joint (double-stream) transformer block built from the library's entry points.
+
+Mirrors `JointTransformerBlock` (Models/Flux1.swift:149-290) for the configuration the hot path is quoted on:
+`contextBlockPreOnly: false`, `upcast: false`, attention level `.scaleMerged`.  The reference graph runs about fifty ops
+per block; here a block is twelve launches:
+
+  2  LayerNorm + modulation of the two fp32 streams                       (dt_layernorm_modulate_f16)
+  1  c_q c_k c_v x_q x_k x_v with per-head RMSNorm and RoPE in the epilogue, written straight into the joint
+     [t + hw, 3, h, k] buffer (no concat)                                   (dt_dense_qx_grouped_f16)
+  1  attention over the joint sequence                                      (dt_sdpa_f16)
+  1  c_o and x_o with gate and fp32 residual accumulation in the epilogue  (dt_dense_qx_grouped_f16 + post)
+  2  LayerNorm + modulation
+  1  c_linear1 and x_linear1 with GELU(tanh)
+  1  c_out_proj and x_out_proj with gate and residual accumulation
+"""
+from typing import Dict, Optional, Sequence
+
+import numpy as np
+
+from . import (ACT_GELU_TANH, DensePost, HeadEpilogue, QxTensor, dense_grouped, layernorm_modulate, sdpa_segments,
+               _torch)
+
+DENSE_NAMES = ("c_q", "c_k", "c_v", "x_q", "x_k", "x_v", "c_o", "x_o", "c_linear1", "c_out_proj", "x_linear1",
+               "x_out_proj")
+NORM_NAMES = ("c_norm_q", "c_norm_k", "x_norm_q", "x_norm_k")
+
+
+class JointTransformerBlock:
+    """k = head dimension, h = heads, t = text tokens, hw = image tokens (batch 1).  `weight[name]` is a QxTensor
+    [out, in], `bias[name]` an fp16 vector, `norm[name]` the fp16 RMSNorm weight [k]."""
+
+    def __init__(self, k: int, h: int, t: int, hw: int):
+        self.k, self.h, self.t, self.hw = k, h, t, hw
+        self.weight: Dict[str, QxTensor] = {}
+        self.bias: Dict[str, object] = {}
+        self.norm: Dict[str, object] = {}
+        self._buffers = None
+
+    def _alloc(self, device):
+        torch = _torch()
+        if self._buffers is None or self._buffers["qkv"].device != device:
+            S, C = self.t + self.hw, self.h * self.k
+            f16 = dict(dtype=torch.float16, device=device)
+            self._buffers = dict(
+                qkv=torch.empty((S, 3, self.h, self.k), **f16), att=torch.empty((1, S, self.h, self.k), **f16),
+                cn=torch.empty((self.t, C), **f16), xn=torch.empty((self.hw, C), **f16),
+                ch=torch.empty((self.t, 4 * C), **f16), xh=torch.empty((self.hw, 4 * C), **f16))
+        return self._buffers
+
+    def __call__(self, context, x, rot, contextChunks: Sequence[object], xChunks: Sequence[object], stream=None):
+        """context [1, t, h k] and x [1, hw, h k] fp32, rot [t + hw, k] fp16 (interleaved cos / sin), the six
+        modulation vectors of each stream fp16 [h k] (shift, scale, gate for attention, then for the feed-forward;
+        the scale already carries its + 1, as the fixed encoder stores it).  Returns the new (context, x), fp32."""
+        torch = _torch()
+        k, h, t, hw = self.k, self.h, self.t, self.hw
+        S, C = t + hw, h * k
+        if tuple(context.shape[-2:]) != (t, C) or tuple(x.shape[-2:]) != (hw, C):
+            raise ValueError("context / x do not match the block's token counts and width")
+        if len(contextChunks) != 6 or len(xChunks) != 6:
+            raise ValueError("six modulation vectors per stream")
+        W, Bv, G = self.weight, self.bias, self.norm
+        buf = self._alloc(x.device)
+        qkv, att, cn, xn = buf["qkv"], buf["att"], buf["cn"], buf["xn"]
+        c_res = context.reshape(t, C).clone()
+        x_res = x.reshape(hw, C).clone()
+        # attention half
+        layernorm_modulate(c_res, contextChunks[1], contextChunks[0], 1e-6, out=cn, stream=stream)
+        layernorm_modulate(x_res, xChunks[1], xChunks[0], 1e-6, out=xn, stream=stream)
+        qkv2 = qkv.view(S, 3 * C)
+        views = lambda lo, hi: [qkv2[lo:hi, i * C:(i + 1) * C] for i in range(3)]
+        epi = lambda q, kk, pos: [HeadEpilogue(G[q], rot, pos, 1e-6, k), HeadEpilogue(G[kk], rot, pos, 1e-6, k), None]
+        dense_grouped([
+            dict(x=xn, weights=[W["x_q"], W["x_k"], W["x_v"]], biases=[Bv["x_q"], Bv["x_k"], Bv["x_v"]],
+                 outs=views(t, S), epilogues=epi("x_norm_q", "x_norm_k", t)),
+            dict(x=cn, weights=[W["c_q"], W["c_k"], W["c_v"]], biases=[Bv["c_q"], Bv["c_k"], Bv["c_v"]],
+                 outs=views(0, t), epilogues=epi("c_norm_q", "c_norm_k", 0))], stream=stream)
+        sdpa_segments([qkv[:, 0].unsqueeze(0)], [qkv[:, 1].unsqueeze(0)], [qkv[:, 2].unsqueeze(0)],
+                      1.0 / float(np.sqrt(k)), out=att, stream=stream)
+        att2 = att.view(S, C)
+        tail = lambda gate, res: [DensePost(gate=gate, residual=res, keep_output=False)]
+        dense_grouped([
+            dict(x=att2[t:], weights=[W["x_o"]], biases=[Bv["x_o"]], posts=tail(xChunks[2], x_res)),
+            dict(x=att2[:t], weights=[W["c_o"]], biases=[Bv["c_o"]], posts=tail(contextChunks[2], c_res))],
+            stream=stream)
+        # feed-forward half
+        layernorm_modulate(c_res, contextChunks[4], contextChunks[3], 1e-6, out=cn, stream=stream)
+        layernorm_modulate(x_res, xChunks[4], xChunks[3], 1e-6, out=xn, stream=stream)
+        gelu = [DensePost(ACT_GELU_TANH)]
+        dense_grouped([
+            dict(x=xn, weights=[W["x_linear1"]], biases=[Bv["x_linear1"]], outs=[buf["xh"]], posts=gelu),
+            dict(x=cn, weights=[W["c_linear1"]], biases=[Bv["c_linear1"]], outs=[buf["ch"]], posts=gelu)],
+            stream=stream)
+        dense_grouped([
+            dict(x=buf["xh"], weights=[W["x_out_proj"]], biases=[Bv["x_out_proj"]], posts=tail(xChunks[5], x_res)),
+            dict(x=buf["ch"], weights=[W["c_out_proj"]], biases=[Bv["c_out_proj"]],
+                 posts=tail(contextChunks[5], c_res))], stream=stream)
+        return c_res.reshape(context.shape), x_res.reshape(x.shape)

@@ -226,7 +226,8 @@ typedef struct {
   const uint16_t* const* bias;
   uint16_t* const* Y;
   const int64_t* ldy;
-  const dt_head_epilogue* epi;
+  const dt_head_epilogue* epi;  /* as for dt_dense_qx_heads_f16, or NULL */
+  const dt_dense_post* post;    /* as for dt_dense_qx_post_f16, or NULL; a problem has at most one of epi and post */
 } dt_dense_group;
 
 dt_status dt_dense_qx_grouped_f16(dt_stream stream, int32_t n_groups, const dt_dense_group* groups,

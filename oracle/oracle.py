@@ -401,3 +401,33 @@ def np_gated_residual(res32: np.ndarray, y16: np.ndarray, gate16=None) -> np.nda
     """res + float32(fp16(y * gate)); gate broadcast over rows."""
     y = y16 if gate16 is None else (y16.astype(np.float32) * gate16.astype(np.float32)[None, :]).astype(np.float16)
     return (res32.astype(np.float32) + y.astype(np.float32)).astype(np.float32)
+
+
+def np_flux_joint_block(context32, x32, rot16, cch, xch, dense, bias, norm, k, h):
+    """Flux.1 JointTransformerBlock op by op (Models/Flux1.swift:149-290; contextBlockPreOnly false, upcast false):
+    LayerNorm + modulation (:160, 172-173), the six projections (:161-183), per-head RMSNorm of Q and K (:164-169,
+    177-182), concat text || image and RoPE (:184-188), attention at scale 1 / sqrt(k) (:228-232), c_o / x_o and the
+    gated residual additions (:236-250), the feed-forward with GELU(tanh) and its gated residual (:130-147, 251-283).
+    `dense[name]` is a callable X16 -> Y16 (this module's Dense with that layer's weight and bias); `norm[name]` the
+    fp16 RMSNorm weight; `cch` / `xch` the six fp16 modulation vectors of each stream.  fp32 streams in and out."""
+    t, hw = context32.shape[0], x32.shape[0]
+    c = np_layernorm_modulate16(context32, cch[1], cch[0], 1e-6, "f16")
+    xx = np_layernorm_modulate16(x32, xch[1], xch[0], 1e-6, "f16")
+    heads = lambda y, n: y.reshape(n, h, k)
+    cK = C.rmsnorm(heads(dense["c_k"](c), t), norm["c_norm_k"], 1e-6)
+    cQ = C.rmsnorm(heads(dense["c_q"](c), t), norm["c_norm_q"], 1e-6)
+    cV = heads(dense["c_v"](c), t)
+    xK = C.rmsnorm(heads(dense["x_k"](xx), hw), norm["x_norm_k"], 1e-6)
+    xQ = C.rmsnorm(heads(dense["x_q"](xx), hw), norm["x_norm_q"], 1e-6)
+    xV = heads(dense["x_v"](xx), hw)
+    keys = C.cmul(np.concatenate([cK, xK], axis=0), rot16)
+    queries = C.cmul(np.concatenate([cQ, xQ], axis=0), rot16)
+    values = np.concatenate([cV, xV], axis=0)
+    out = C.sdpa(queries[None], keys[None], values[None], 1.0 / np.sqrt(k))[0].reshape(t + hw, h * k)
+    context = np_gated_residual(context32, dense["c_o"](np.ascontiguousarray(out[:t])), cch[2])
+    x = np_gated_residual(x32, dense["x_o"](np.ascontiguousarray(out[t:])), xch[2])
+    ff = lambda y, name: dense[name + "_out_proj"](np_gelu_tanh16(dense[name + "_linear1"](y)))
+    context = np_gated_residual(context, ff(np_layernorm_modulate16(context, cch[4], cch[3], 1e-6, "f16"), "c"), cch[5])
+    x = np_gated_residual(x, ff(np_layernorm_modulate16(x, xch[4], xch[3], 1e-6, "f16"), "x"), xch[5])
+    return context, x
+
