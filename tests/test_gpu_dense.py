@@ -427,6 +427,53 @@ def test_lora_dense(dthip, oracle, torch_cuda, M, N, K, q, nib, rank, scale):
     assert torch.equal(plain(xd), base)
 
 
+def test_dense_grouped_with_tails_equals_separate(dthip, oracle, torch_cuda):
+    """Problems that carry elementwise tails share a launch like plain ones (c_o / x_o with gate and residual,
+    c_linear1 / x_linear1 with GELU): bit-identical to one dt_dense_qx_post_f16 call per problem, for the fused launch
+    (a problem with M >= 1024), the problem-by-problem route (small M) and a mix of a tail problem with a head-epilogue
+    problem, which must not share a launch."""
+    torch = torch_cuda
+    rng = np.random.default_rng(77)
+    K, N, q, nib = 256, 384, 6, 4096
+    for Ms in ((1100, 200), (150, 60)):
+        print("dense grouped tails", Ms, flush=True)
+        xs = [to_dev(torch, rng.standard_normal((M, K)).astype(np.float16)) for M in Ms]
+        ws = [make_weight(dthip, oracle, rng, N, K, q, nib, std=0.05)[0] for _ in Ms]
+        bs = [to_dev(torch, (rng.standard_normal(N) * 0.1).astype(np.float16)) for _ in Ms]
+        gates = [to_dev(torch, (1 + 0.3 * rng.standard_normal(N)).astype(np.float16)) for _ in Ms]
+        res0 = [torch.randn((M, N), dtype=torch.float32, device="cuda") for M in Ms]
+        # gate + residual, accumulate only
+        want = [r.clone() for r in res0]
+        for x, w, b, g, r in zip(xs, ws, bs, gates, want):
+            assert dthip.dense_post(x, [w], [b], [dthip.DensePost(gate=g, residual=r, keep_output=False)])[0] is None
+        got = [r.clone() for r in res0]
+        outs = dthip.dense_grouped([dict(x=x, weights=[w], biases=[b],
+                                         posts=[dthip.DensePost(gate=g, residual=r, keep_output=False)])
+                                    for x, w, b, g, r in zip(xs, ws, bs, gates, got)])
+        assert all(o == [None] for o in outs)
+        assert all(torch.equal(a, b) for a, b in zip(got, want))
+        assert not torch.equal(got[0], res0[0])
+        # GELU with the fp16 result kept
+        want = [dthip.dense_post(x, [w], [b], [dthip.DensePost(dthip.ACT_GELU_TANH)])[0] for x, w, b in zip(xs, ws, bs)]
+        outs = dthip.dense_grouped([dict(x=x, weights=[w], biases=[b], posts=[dthip.DensePost(dthip.ACT_GELU_TANH)])
+                                    for x, w, b in zip(xs, ws, bs)])
+        assert all(torch.equal(o[0], wv) for o, wv in zip(outs, want))
+    # a tail problem next to a head-epilogue problem
+    M, D = 1100, 128
+    x = to_dev(torch, rng.standard_normal((M, K)).astype(np.float16))
+    wh, _ = make_weight(dthip, oracle, rng, 2 * D, K, q, nib, std=0.05)
+    gamma = to_dev(torch, (1 + 0.1 * rng.standard_normal(D)).astype(np.float16))
+    epi = dthip.HeadEpilogue(gamma, None, 0, 1e-6, D)
+    want_h = dthip.dense_multi(x, [wh], [None], epilogues=[epi])[0]
+    want_t = dthip.dense_post(xs[0][:100], [ws[0]], [bs[0]], [dthip.DensePost(dthip.ACT_SWISH)])[0]
+    outs = dthip.dense_grouped([dict(x=x, weights=[wh], biases=[None], epilogues=[epi]),
+                                dict(x=xs[0][:100], weights=[ws[0]], biases=[bs[0]], posts=[dthip.DensePost(dthip.ACT_SWISH)])])
+    assert torch.equal(outs[0][0], want_h) and torch.equal(outs[1][0], want_t)
+    # a problem may not carry both
+    with pytest.raises(dthip.DtError):
+        dthip.dense_grouped([dict(x=x, weights=[wh], biases=[None], epilogues=[epi], posts=[dthip.DensePost()])])
+
+
 def test_dense_post_bad_args(dthip, oracle, torch_cuda):
     torch = torch_cuda
     rng = np.random.default_rng(9)
