@@ -64,7 +64,7 @@ class _HeadEpilogue(ctypes.Structure):
 class _DensePost(ctypes.Structure):
     _fields_ = [("activation", ctypes.c_int32), ("gate", ctypes.c_void_p), ("residual", ctypes.c_void_p),
                 ("ld_residual", ctypes.c_int64), ("scale", ctypes.c_float), ("addend", ctypes.c_void_p),
-                ("ld_addend", ctypes.c_int64)]
+                ("ld_addend", ctypes.c_int64), ("gate_f32", ctypes.c_void_p)]
 
 
 class _DenseGroup(ctypes.Structure):
@@ -359,8 +359,9 @@ ACT_NONE, ACT_GELU_TANH, ACT_SWISH = 0, 1, 2
 class DensePost:
     """Elementwise tail of one projection, in this order: scalar `scale`, fp16 `addend` [M, N] (the low-rank branch of a
     LoRADense, Models/LoRA.swift:117-140), activation (ACT_*), per-feature fp16 gate [N], fp32 residual [M, N] that the
-    result is accumulated into (`x + (y .* gate).to(of: x)`, Models/Flux1.swift:250).  With `residual` given and
-    `keep_output=False` the fp16 result itself is not written."""
+    result is accumulated into (`x + (y .* gate).to(of: x)`, Models/Flux1.swift:250).  A float32 gate multiplies in
+    fp32 on the way into the residual instead (`x + out.to(of: x) .* chunks[2]`, Models/Wan.swift:159).  With
+    `residual` given and `keep_output=False` the fp16 result itself is not written."""
 
     def __init__(self, activation: int = ACT_NONE, gate=None, residual=None, keep_output: bool = True,
                  scale: float = 1.0, addend=None):
@@ -375,11 +376,19 @@ def _marshal_posts(posts, weights, M, Y, outs):
     P = (_DensePost * n)()
     for i, p in enumerate(posts):
         if p is None:
-            P[i] = _DensePost(ACT_NONE, None, None, 0, 1.0, None, 0)
+            P[i] = _DensePost(ACT_NONE, None, None, 0, 1.0, None, 0, None)
             continue
         N = weights[i].shape[0]
-        if p.gate is not None and (_f16_cuda(p.gate, "gate").numel() != N or not p.gate.is_contiguous()):
-            raise ValueError("gate must hold one value per output feature")
+        g16 = g32 = None
+        if p.gate is not None:
+            if isinstance(p.gate, torch.Tensor) and p.gate.dtype == torch.float32:  # product formed in fp32 (Wan)
+                if not p.gate.is_cuda:
+                    raise TypeError("gate must be a CUDA tensor")
+                g32 = p.gate
+            else:
+                g16 = _f16_cuda(p.gate, "gate")
+            if p.gate.numel() != N or not p.gate.is_contiguous():
+                raise ValueError("gate must hold one value per output feature")
         rp, ldr = None, 0
         if p.residual is not None:
             r = p.residual
@@ -399,7 +408,8 @@ def _marshal_posts(posts, weights, M, Y, outs):
             if a2.shape != (M, N) or a2.stride(1) != 1 or a2.data_ptr() != p.addend.data_ptr():
                 raise ValueError("addend must be an [M, N] view with contiguous rows")
             ap, lda = a2.data_ptr(), a2.stride(0)
-        P[i] = _DensePost(p.activation, None if p.gate is None else p.gate.data_ptr(), rp, ldr, float(p.scale), ap, lda)
+        P[i] = _DensePost(p.activation, None if g16 is None else g16.data_ptr(), rp, ldr, float(p.scale), ap, lda,
+                          None if g32 is None else g32.data_ptr())
     return P
 
 
@@ -559,13 +569,14 @@ class RMSNorm:
         raise DtError("RMSNorm", DT_NO_KERNEL)
 
 
-MOD_F16, MOD_F32 = 0, 1
+MOD_F16, MOD_F32, MOD_AFFINE_F32 = 0, 1, 2
 
 
-def layernorm_modulate(x, scale=None, shift=None, epsilon: float = 1e-6, out=None, stream=None):
+def layernorm_modulate(x, scale=None, shift=None, epsilon: float = 1e-6, out=None, stream=None, affine: bool = False):
     """LayerNorm(epsilon:, axis: [last], elementwiseAffine: false) of the fp32 stream `x` [..., C], then the adaLN
     modulation, fp16 out.  fp16 `scale` / `shift` [C]: `norm(x).to(.Float16) .* scale + shift` (Models/Flux1.swift:
-    172-173); fp32 ones: `(norm(x) .* (scale + 1) + shift).to(.Float16)` (Models/Wan.swift:217-221)."""
+    172-173); fp32 ones: `(norm(x) .* (scale + 1) + shift).to(.Float16)` (Models/Wan.swift:217-221), or with
+    `affine=True` the LayerNorm's own fp32 weight and bias, `norm(x) * scale + shift` (Models/Wan.swift:160-161)."""
     torch = _torch()
     if not (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.float32):
         raise TypeError("x must be a float32 CUDA tensor")
@@ -582,6 +593,10 @@ def layernorm_modulate(x, scale=None, shift=None, epsilon: float = 1e-6, out=Non
         if not t.is_cuda or t.numel() != C or not t.is_contiguous():
             raise ValueError("scale / shift must be contiguous CUDA vectors of C elements")
     mod = MOD_F32 if dtypes == {torch.float32} else MOD_F16
+    if affine:
+        if mod != MOD_F32:
+            raise TypeError("affine LayerNorm takes float32 weight and bias")
+        mod = MOD_AFFINE_F32
     if out is None:
         out = torch.empty((M, C), dtype=torch.float16, device=x.device)
     elif out.dtype != torch.float16 or out.shape != (M, C) or out.stride(1) != 1:
@@ -595,18 +610,23 @@ def layernorm_modulate(x, scale=None, shift=None, epsilon: float = 1e-6, out=Non
 
 
 class LayerNorm:
-    """LayerNorm(epsilon:axis:elementwiseAffine: false) on the last axis of an fp32 tensor, result cast to fp16
-    (`xNorm1(x).to(.Float16)`, Models/Flux1.swift:172-173).  The affine form is not on the accelerated path."""
+    """LayerNorm(epsilon:axis:elementwiseAffine:) on the last axis of an fp32 tensor, result cast to fp16
+    (`xNorm1(x).to(.Float16)`, Models/Flux1.swift:172-173; with fp32 `weight` / `bias` `xNorm3(out).to(.Float16)`,
+    Models/Wan.swift:160-161)."""
 
     def __init__(self, epsilon: float, axis: Sequence[int], elementwiseAffine: bool = True, name: str = ""):
-        if elementwiseAffine:
-            raise NotImplementedError("LayerNorm with elementwiseAffine is not provided")
-        self.epsilon, self.axis, self.name = epsilon, list(axis), name
+        self.epsilon, self.axis, self.elementwiseAffine, self.name = epsilon, list(axis), elementwiseAffine, name
+        self.weight = None
+        self.bias = None
 
     def __call__(self, x, stream=None):
         if self.axis != [x.dim() - 1]:
             raise ValueError("LayerNorm: only the last axis is supported")
-        return layernorm_modulate(x, None, None, self.epsilon, stream=stream)
+        if not self.elementwiseAffine:
+            return layernorm_modulate(x, None, None, self.epsilon, stream=stream)
+        if self.weight is None or self.bias is None:
+            raise RuntimeError(f"LayerNorm {self.name!r}: weight / bias not loaded")
+        return layernorm_modulate(x, self.weight, self.bias, self.epsilon, stream=stream, affine=True)
 
 
 def _as_heads(y):

@@ -18,6 +18,7 @@ __device__ __forceinline__ float round16(float v) { return (float)(half_t)v; }
 // One normalised value through the modulation (sc, sh already widened to float).
 //   DT_MOD_F16: fp16(fp16(fp16(n) * scale) + shift), scale and shift fp16
 //   DT_MOD_F32: fp16(n * (scale + 1) + shift), scale and shift fp32
+//   DT_MOD_AFFINE_F32: fp16(n * scale + shift), scale and shift fp32
 template <int MOD>
 __device__ __forceinline__ uint16_t modulate(float n, bool has_scale, float sc, bool has_shift, float sh) {
   if constexpr (MOD == DT_MOD_F16) {
@@ -25,7 +26,7 @@ __device__ __forceinline__ uint16_t modulate(float n, bool has_scale, float sc, 
     if (has_scale) n = round16(n * sc);
     if (has_shift) n = round16(n + sh);
   } else {
-    if (has_scale) n = n * (sc + 1.0f);
+    if (has_scale) n = n * (MOD == DT_MOD_F32 ? sc + 1.0f : sc);
     if (has_shift) n = n + sh;
   }
   return half_to_bits((half_t)n);
@@ -154,7 +155,7 @@ DT_EXPORT dt_status dt_layernorm_modulate_f16(dt_stream stream, int64_t M, int64
                                               const void* scale, const void* shift, int32_t mod, float eps,
                                               uint16_t* Y, int64_t ldy) {
   using namespace dt;
-  if (M < 0 || C <= 0 || (mod != DT_MOD_F16 && mod != DT_MOD_F32)) return DT_INVALID;
+  if (M < 0 || C <= 0 || mod < DT_MOD_F16 || mod > DT_MOD_AFFINE_F32) return DT_INVALID;
   if (!(eps >= 0.f) || eps - eps != 0.f) return DT_INVALID;
   if (M == 0) return DT_OK;
   if (!X || !Y || ldx < C || ldy < C) return DT_INVALID;
@@ -169,6 +170,7 @@ DT_EXPORT dt_status dt_layernorm_modulate_f16(dt_stream stream, int64_t M, int64
                    (reinterpret_cast<uintptr_t>(scale) & (mod == DT_MOD_F16 ? 7 : 15)) == 0 &&
                    (reinterpret_cast<uintptr_t>(shift) & (mod == DT_MOD_F16 ? 7 : 15)) == 0;
   if (mod == DT_MOD_F16) launch_adaln<DT_MOD_F16>(as_stream(stream), a, vec);
-  else launch_adaln<DT_MOD_F32>(as_stream(stream), a, vec);
+  else if (mod == DT_MOD_F32) launch_adaln<DT_MOD_F32>(as_stream(stream), a, vec);
+  else launch_adaln<DT_MOD_AFFINE_F32>(as_stream(stream), a, vec);
   return launch_status();
 }

@@ -51,6 +51,7 @@ struct DenseWeight {
   const uint16_t* gate;  // [n] or null
   float* res;            // [m, n] fp32 with row stride ld_res, updated in place; null = none
   int64_t ld_res;
+  const float* gate32;   // [n] fp32 or null: the residual receives float(result) * gate32 (no fp16 product)
 };
 
 // The elementwise tail on one value that has already been rounded to fp16, with
@@ -589,7 +590,8 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       uint16_t* yrow = w.y ? w.y + gmc * w.ldy : nullptr;
       float* rrow = w.res ? w.res + gmc * w.ld_res : nullptr;
       const uint16_t* arow = w.add ? w.add + gmc * w.ld_add : nullptr;
-      const bool vec = (!w.add || (((w.ld_add & 3) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 7) == 0)) &&
+      const bool vec = (!w.gate32 || (reinterpret_cast<uintptr_t>(w.gate32) & 15) == 0) &&
+                       (!w.add || (((w.ld_add & 3) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 7) == 0)) &&
                        (!w.gate || (reinterpret_cast<uintptr_t>(w.gate) & 7) == 0) &&
                        (!w.bias || (reinterpret_cast<uintptr_t>(w.bias) & 7) == 0) &&
                        (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0)) &&
@@ -600,7 +602,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         for (int gq = 0; gq < 4; gq++) {
           const int nn = n0 + wn * WN + i * 32 + 8 * gq + 4 * hi;
           float bq[4] = {0.f, 0.f, 0.f, 0.f}, gt[4] = {1.f, 1.f, 1.f, 1.f}, rr[4] = {0.f, 0.f, 0.f, 0.f}, pv[4];
-          float ad[4] = {0.f, 0.f, 0.f, 0.f};
+          float ad[4] = {0.f, 0.f, 0.f, 0.f}, g32[4] = {1.f, 1.f, 1.f, 1.f};
           const bool full = vec && nn + 3 < w.n;
           if (gm < g.m) {
             if (full) {
@@ -613,6 +615,10 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
                 const uint2_t t2 = *reinterpret_cast<const uint2_t*>(w.gate + nn);
                 gt[0] = (float)bits_to_half((uint16_t)t2[0]); gt[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
                 gt[2] = (float)bits_to_half((uint16_t)t2[1]); gt[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
+              }
+              if (w.gate32) {
+                const float4_t t4 = *reinterpret_cast<const float4_t*>(w.gate32 + nn);
+                g32[0] = t4[0]; g32[1] = t4[1]; g32[2] = t4[2]; g32[3] = t4[3];
               }
               if (arow) {
                 const uint2_t t2 = *reinterpret_cast<const uint2_t*>(arow + nn);
@@ -631,13 +637,16 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
                   if (w.gate) gt[e] = (float)bits_to_half(w.gate[nn + e]);
                   if (rrow) rr[e] = rrow[nn + e];
                   if (arow) ad[e] = (float)bits_to_half(arow[nn + e]);
+                  if (w.gate32) g32[e] = w.gate32[nn + e];
                 }
             }
 #pragma unroll
             for (int e = 0; e < 4; e++) {
               const float v0 = (float)(half_t)(acc[i][j][4 * gq + e] + bq[e]);
               pv[e] = post_value(v0, w.scale, arow != nullptr, ad[e], w.act, w.gate != nullptr, gt[e]);
-              rr[e] += pv[e];
+              float pr = pv[e] * g32[e];  // the product is its own op: rounded before the addition
+              asm volatile("" : "+v"(pr));
+              rr[e] += pr;
             }
             if (full) {
               if (rrow) *reinterpret_cast<float4_t*>(rrow + nn) = float4_t{rr[0], rr[1], rr[2], rr[3]};
@@ -816,7 +825,7 @@ __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* _
                                                              uint16_t* y, int64_t ldy, float scale,
                                                              const uint16_t* add, int64_t ld_add, int act,
                                                              const uint16_t* __restrict__ gate, float* __restrict__ res,
-                                                             int64_t ld_res) {
+                                                             int64_t ld_res, const float* __restrict__ gate32) {
   int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (o >= m * n) return;
   int64_t mi = o / n, ni = o - mi * n;
@@ -840,7 +849,11 @@ __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* _
   float v = (float)(half_t)acc;
   v = post_value(v, scale, add != nullptr, add ? (float)bits_to_half(add[mi * ld_add + ni]) : 0.f, act, gate != nullptr,
                  gate ? (float)bits_to_half(gate[ni]) : 1.0f);
-  if (res) res[mi * ld_res + ni] += v;
+  if (res) {
+    float pr = gate32 ? v * gate32[ni] : v;
+    asm volatile("" : "+v"(pr));  // no fused multiply-add: the product is rounded first
+    res[mi * ld_res + ni] += pr;
+  }
   if (y) y[mi * ldy + ni] = half_to_bits((half_t)v);
 }
 
@@ -954,6 +967,7 @@ static dt_status validate_group(const HostGroup& h) {
       if (p.addend && ((reinterpret_cast<uintptr_t>(p.addend) & 1) || (h.W && h.K > 0 && p.ld_addend < h.W[i].count / h.K)))
         return DT_INVALID;
       if (!(p.scale == p.scale) || p.scale - p.scale != 0.f) return DT_INVALID;  // NaN or infinite
+      if (p.gate_f32 && (!p.residual || p.gate || (reinterpret_cast<uintptr_t>(p.gate_f32) & 3))) return DT_INVALID;
     }
   if (h.M > 0x7fffffff || h.K > 0x7fffffff) return DT_INVALID;
   for (int i = 0; i < h.n_weights; i++) {
@@ -1014,6 +1028,7 @@ static int add_weight(DenseArgs& a, int slot, const HostGroup& h, int wi, int ti
   d.gate = h.post ? h.post[wi].gate : nullptr;
   d.res = h.post ? h.post[wi].residual : nullptr;
   d.ld_res = h.post ? h.post[wi].ld_residual : 0;
+  d.gate32 = h.post ? h.post[wi].gate_f32 : nullptr;
   return (int)((n_rows + BN - 1) / BN);
 }
 
@@ -1046,7 +1061,7 @@ static dt_status run_group(hipStream_t s, const HostGroup& h) {
                            h.post ? h.post[i].addend : nullptr, h.post ? h.post[i].ld_addend : 0,
                            h.post ? h.post[i].activation : DT_ACT_NONE,
                            h.post ? h.post[i].gate : nullptr, h.post ? h.post[i].residual : nullptr,
-                           h.post ? h.post[i].ld_residual : 0);
+                           h.post ? h.post[i].ld_residual : 0, h.post ? h.post[i].gate_f32 : nullptr);
         dt_status st = launch_status();
         if (st != DT_OK) return st;
         if (h.wants_epi(i)) {

@@ -161,6 +161,9 @@ dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K, const ui
  *   gate       : [N_i] fp16, multiplies every output row ((xOut .* xChunks[2]), Models/Flux1.swift:246-250)
  *   residual   : fp32 [M, N_i] with row stride ld_residual, updated in place:
  *                residual += float(result)  (x + (...).to(of: x), Models/Flux1.swift:250, 275-283)
+ *   gate_f32   : [N_i] fp32, needs residual, excludes gate: residual += float(result) * gate_f32, the product
+ *                formed in fp32 (x + out.to(of: x) .* chunks[2], Models/Wan.swift:159, 220-221); Y[i], if given,
+ *                receives the result before the gate
  * post: HOST array of n_weights entries (NULL = plain dt_dense_qx_f16).  Y[i] may
  * be NULL when post[i].residual is given (the result is only accumulated).
  * Concurrent calls must not share a residual tensor.
@@ -177,6 +180,7 @@ typedef struct {
   float scale;
   const uint16_t* addend;
   int64_t ld_addend;
+  const float* gate_f32;
 } dt_dense_post;
 
 dt_status dt_dense_qx_post_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,
@@ -192,6 +196,8 @@ dt_status dt_dense_qx_post_f16(dt_stream stream, int64_t M, int64_t K, const uin
  *                (xNorm1(x).to(.Float16) .* xChunks[1] + xChunks[0], Models/Flux1.swift:172-173, 281-282)
  *   DT_MOD_F32 : y = fp16(norm(x) * (scale + 1) + shift), scale / shift fp32 [C]
  *                ((xNorm2(out) .* (chunks[4] + 1) + chunks[3]).to(.Float16), Models/Wan.swift:217-221)
+ *   DT_MOD_AFFINE_F32 : y = fp16(norm(x) * scale + shift), scale / shift fp32 [C]: LayerNorm with its
+ *                elementwise affine weight and bias (xNorm3(out).to(.Float16), Models/Wan.swift:160-161)
  * norm(x) = (x - mean) / sqrt(var + eps) with the biased variance, in fp32.
  * X: [M, C] fp32 with row stride ldx; Y: [M, C] fp16 with row stride ldy; scale
  * and shift are broadcast over rows and may be NULL.  Rows that are 16-byte
@@ -200,6 +206,7 @@ dt_status dt_dense_qx_post_f16(dt_stream stream, int64_t M, int64_t K, const uin
  */
 #define DT_MOD_F16 0
 #define DT_MOD_F32 1
+#define DT_MOD_AFFINE_F32 2
 
 dt_status dt_layernorm_modulate_f16(dt_stream stream, int64_t M, int64_t C, const float* X, int64_t ldx,
                                     const void* scale, const void* shift, int32_t mod, float eps,

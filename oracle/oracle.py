@@ -363,6 +363,7 @@ def np_layernorm_modulate16(x32: np.ndarray, scale=None, shift=None, eps: float 
     out.  mod "f16": fp16(fp16(fp16(norm) * scale) + shift) with fp16 scale / shift -- xNorm1(x).to(.Float16) .*
     xChunks[1] + xChunks[0] (Models/Flux1.swift:172-173, 281-282).  mod "f32": fp16(norm * (scale + 1) + shift) with
     fp32 scale / shift -- (xNorm2(out) .* (chunks[4] + 1) + chunks[3]).to(.Float16) (Models/Wan.swift:217-221).
+    mod "affine": fp16(norm * scale + shift), the LayerNorm's own fp32 weight and bias (Models/Wan.swift:160-161).
     Statistics in float64 (biased variance), the normalised value rounded to float32 as the fp32 op leaves it."""
     x = x32.astype(np.float64)
     mean = x.mean(axis=-1, keepdims=True)
@@ -376,7 +377,7 @@ def np_layernorm_modulate16(x32: np.ndarray, scale=None, shift=None, eps: float 
             y = (y.astype(np.float32) + shift.astype(np.float16).astype(np.float32)).astype(np.float16)
         return y
     if scale is not None:
-        n = n * (scale.astype(np.float32) + np.float32(1))
+        n = n * (scale.astype(np.float32) + np.float32(1) if mod == "f32" else scale.astype(np.float32))
     if shift is not None:
         n = n + shift.astype(np.float32)
     return n.astype(np.float16)
@@ -395,6 +396,15 @@ def np_add16(a16: np.ndarray, b16: np.ndarray) -> np.ndarray:
     """fp16 elementwise sum (out = dense(x) + up(...), Models/LoRA.swift:128-140); the float32 sum of two fp16 values
     is exact, so one rounding."""
     return (a16.astype(np.float32) + b16.astype(np.float32)).astype(np.float16)
+
+
+def np_gated_residual32(res32: np.ndarray, y16: np.ndarray, gate32=None) -> np.ndarray:
+    """res + float32(y) * gate32, the product formed in fp32 (x + out.to(of: x) .* chunks[2], Models/Wan.swift:159,
+    220-221); gate broadcast over rows."""
+    y = y16.astype(np.float32)
+    if gate32 is not None:
+        y = y * gate32.astype(np.float32)[None, :]
+    return (res32.astype(np.float32) + y).astype(np.float32)
 
 
 def np_gated_residual(res32: np.ndarray, y16: np.ndarray, gate16=None) -> np.ndarray:
@@ -430,4 +440,33 @@ def np_flux_joint_block(context32, x32, rot16, cch, xch, dense, bias, norm, k, h
     context = np_gated_residual(context, ff(np_layernorm_modulate16(context, cch[4], cch[3], 1e-6, "f16"), "c"), cch[5])
     x = np_gated_residual(x, ff(np_layernorm_modulate16(x, xch[4], xch[3], 1e-6, "f16"), "x"), xch[5])
     return context, x
+
+
+def np_wan_attention_block(x32, rot16, chunks32, cK16, cV16, dense, norm, norm3_w32, norm3_b32, k, h):
+    """WanAttentionBlock op by op (Models/Wan.swift:68-277; batch 1, no causal inference, no injected image,
+    self-attention at level .scale1): LayerNorm + fp32 modulation (:81-82), x_q / x_k / x_v with whole-row RMSNorm on Q
+    and K (:83-92), RoPE (:93-94), the k^(-1/4) scale on both (:95-98), attention at scale 1 (:103, 129-131), x_o and
+    the fp32-gated residual (:157-159), affine LayerNorm x_norm_3 (:160-161), x_c_q with whole-row RMSNorm (:162-167),
+    cross-attention at 1 / sqrt(k) over the given context K / V (:169-174), c_o and its residual (:215-216), the
+    feed-forward and its fp32-gated residual (:217-221).  `chunks32` = c + modulations, six fp32 vectors.
+    `dense[name]`: callable X16 -> Y16; `norm[name]`: fp16 whole-row RMSNorm weights.  fp32 stream in and out."""
+    hw = x32.shape[0]
+    C_ = h * k
+    xn = np_layernorm_modulate16(x32, chunks32[1], chunks32[0], 1e-6, "f32")
+    xK = C.rmsnorm(dense["x_k"](xn), norm["x_norm_k"], 1e-6).reshape(hw, h, k)
+    xQ = C.rmsnorm(dense["x_q"](xn), norm["x_norm_q"], 1e-6).reshape(hw, h, k)
+    xV = dense["x_v"](xn).reshape(hw, h, k)
+    quarter = np.float32(1.0 / np.sqrt(np.sqrt(k)))
+    scale16 = lambda a: (a.astype(np.float32) * quarter).astype(np.float16)
+    queries = scale16(C.cmul(xQ, rot16))
+    keys = scale16(C.cmul(xK, rot16))
+    att = C.sdpa(queries[None], keys[None], xV[None], 1.0)[0].reshape(hw, C_)
+    out = np_gated_residual32(x32, dense["x_o"](att), chunks32[2])
+    xn = np_layernorm_modulate16(out, norm3_w32, norm3_b32, 1e-6, "affine")
+    cQ = C.rmsnorm(dense["x_c_q"](xn), norm["x_c_norm_q"], 1e-6).reshape(hw, h, k)
+    cross = C.sdpa(cQ[None], cK16, cV16, 1.0 / np.sqrt(k))[0].reshape(hw, C_)
+    out = np_gated_residual32(out, dense["c_o"](cross), None)
+    xn = np_layernorm_modulate16(out, chunks32[4], chunks32[3], 1e-6, "f32")
+    ff = dense["x_out_proj"](np_gelu_tanh16(dense["x_linear1"](xn)))
+    return np_gated_residual32(out, ff, chunks32[5])
 

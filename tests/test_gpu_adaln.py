@@ -21,24 +21,25 @@ def close(got, want, shift=None):
 
 
 @pytest.mark.parametrize("M,C", [(7, 256), (300, 3072), (64, 5120), (5, 8192), (9, 1000), (3, 130), (2, 8200), (1, 4)])
-@pytest.mark.parametrize("mod", ["f16", "f32"])
+@pytest.mark.parametrize("mod", ["f16", "f32", "affine"])
 def test_layernorm_modulate_vs_oracle(dthip, oracle, M, C, mod):
     import torch
     rng = np.random.default_rng(M * 31 + C)
     x = (rng.standard_normal((M, C)) * 2 + 0.5).astype(np.float32)
     dt = np.float16 if mod == "f16" else np.float32
-    scale = ((1 if mod == "f16" else 0) + 0.3 * rng.standard_normal(C)).astype(dt)
+    scale = ((0 if mod == "f32" else 1) + 0.3 * rng.standard_normal(C)).astype(dt)
     shift = (0.5 * rng.standard_normal(C)).astype(dt)
     xd, sd, hd = torch.from_numpy(x).cuda(), torch.from_numpy(scale).cuda(), torch.from_numpy(shift).cuda()
     print("adaln", M, C, mod, flush=True)
-    got = dthip.layernorm_modulate(xd, sd, hd, 1e-6).cpu().numpy()
+    aff = mod == "affine"
+    got = dthip.layernorm_modulate(xd, sd, hd, 1e-6, affine=aff).cpu().numpy()
     assert close(got, oracle.np_layernorm_modulate16(x, scale, shift, 1e-6, mod), shift)
     # no modulation, scale only, shift only
     assert close(dthip.layernorm_modulate(xd, None, None, 1e-6).cpu().numpy(),
                  oracle.np_layernorm_modulate16(x, None, None, 1e-6, mod))
-    assert close(dthip.layernorm_modulate(xd, sd, None, 1e-6).cpu().numpy(),
+    assert close(dthip.layernorm_modulate(xd, sd, None, 1e-6, affine=aff).cpu().numpy(),
                  oracle.np_layernorm_modulate16(x, scale, None, 1e-6, mod))
-    assert close(dthip.layernorm_modulate(xd, None, hd, 1e-6).cpu().numpy(),
+    assert close(dthip.layernorm_modulate(xd, None, hd, 1e-6, affine=aff).cpu().numpy(),
                  oracle.np_layernorm_modulate16(x, None, shift, 1e-6, mod), shift)
 
 

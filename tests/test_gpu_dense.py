@@ -469,6 +469,16 @@ def test_dense_grouped_with_tails_equals_separate(dthip, oracle, torch_cuda):
     outs = dthip.dense_grouped([dict(x=x, weights=[wh], biases=[None], epilogues=[epi]),
                                 dict(x=xs[0][:100], weights=[ws[0]], biases=[bs[0]], posts=[dthip.DensePost(dthip.ACT_SWISH)])])
     assert torch.equal(outs[0][0], want_h) and torch.equal(outs[1][0], want_t)
+    # fp32 gate: the residual receives float(result) * gate, the product formed in fp32; exact against numpy
+    g32 = (1 + 0.3 * rng.standard_normal(N)).astype(np.float32)
+    r0 = rng.standard_normal((100, N)).astype(np.float32)
+    r = to_dev(torch, r0)
+    plain = dthip.dense_multi(xs[0][:100], [ws[0]], [bs[0]])[0].cpu().numpy()
+    kept = dthip.dense_post(xs[0][:100], [ws[0]], [bs[0]], [dthip.DensePost(gate=to_dev(torch, g32), residual=r)])[0]
+    assert np.array_equal(kept.cpu().numpy().view(np.uint16), plain.view(np.uint16))  # the output is the ungated result
+    assert np.array_equal(r.cpu().numpy(), oracle.np_gated_residual32(r0, plain, g32))
+    with pytest.raises(dthip.DtError):  # an fp32 gate needs a residual to go into
+        dthip.dense_post(xs[0][:100], [ws[0]], [bs[0]], [dthip.DensePost(gate=to_dev(torch, g32))])
     # a problem may not carry both
     with pytest.raises(dthip.DtError):
         dthip.dense_grouped([dict(x=x, weights=[wh], biases=[None], epilogues=[epi], posts=[dthip.DensePost()])])

@@ -59,3 +59,49 @@ def test_flux_joint_block_vs_oracle(dthip, oracle, h, t, gh, gw, q, nib):
     # the inputs are left untouched and a second call gives the same result
     again_c, again_x = blk(dev(context), dev(x), dev(rot), [dev(v) for v in cch], [dev(v) for v in xch])
     assert torch.equal(again_c, got_c) and torch.equal(again_x, got_x)
+
+
+@pytest.mark.parametrize("h,gt,gh,gw,t,q,nib", [(2, 3, 16, 24, 64, 5, 1024), (1, 2, 6, 10, 40, 6, 64)])
+def test_wan_attention_block_vs_oracle(dthip, oracle, h, gt, gh, gw, t, q, nib):
+    """A whole Wan attention block (self-attention with whole-row RMSNorm, RoPE and the .scale1 convention,
+    cross-attention over fixed context K / V, feed-forward; fp32 modulation and fp32 gates) against the oracle's
+    op-by-op restatement of Models/Wan.swift:68-277.  Same bar as the Flux block."""
+    import torch
+    wan = importlib.import_module(dthip.__name__ + ".wan")
+    k = 128
+    hw, C = gt * gh * gw, h * k
+    inter = 3 * C
+    rng = np.random.default_rng(hw + t)
+    blk = wan.WanAttentionBlock(k, h, hw, inter)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    dense, norm = {}, {}
+    for name in wan.DENSE_NAMES:
+        N, K = (inter, C) if name == "x_linear1" else (C, inter) if name == "x_out_proj" else (C, C)
+        packed, _, _ = oracle.synth_qx_weight(rng, N, K, q, nib, 1.0 / np.sqrt(K))
+        b = (rng.standard_normal(N) * 0.05).astype(np.float16)
+        blk.weight[name] = dthip.QxTensor.from_packed(packed, q, nib, (N, K))
+        blk.bias[name] = dev(b)
+        dense[name] = (lambda p, n, bb: (lambda X: oracle.C.dense_qx(X, p, q, nib, n, bb)))(packed, N, b)
+    for name in wan.ROW_NORM_NAMES:
+        g = (1 + 0.05 * rng.standard_normal(C)).astype(np.float16)
+        blk.norm[name] = dev(g)
+        norm[name] = g
+    n3w = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
+    n3b = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    blk.norm3_weight, blk.norm3_bias = dev(n3w), dev(n3b)
+    mods = [(0.2 * rng.standard_normal(C)).astype(np.float32) for _ in range(6)]
+    cs = [(0.2 * rng.standard_normal(C)).astype(np.float32) for _ in range(6)]
+    blk.modulation = [dev(m) for m in mods]
+    rot = dthip.WanRotaryPositionEmbedding(gh, gw, gt, channels=k).astype(np.float16)
+    assert rot.shape == (hw, k)
+    x = (rng.standard_normal((1, hw, C)) * 2).astype(np.float32)
+    cK = rng.standard_normal((1, t, h, k)).astype(np.float16)
+    cV = rng.standard_normal((1, t, h, k)).astype(np.float16)
+    print("wan block", h, hw, t, q, nib, flush=True)
+    got = blk(dev(x), dev(rot), [dev(c) for c in cs], dev(cK), dev(cV)).cpu().numpy()[0]
+    chunks = [c + m for c, m in zip(cs, mods)]
+    want = oracle.np_wan_attention_block(x[0], rot, chunks, cK, cV, dense, norm, n3w, n3b, k, h)
+    mx, rr = oracle.err_stats(got, want)
+    print("x max-abs", mx, "rel-rms", rr, "scale", float(np.abs(want).max()), flush=True)
+    assert mx <= 2e-2 and rr <= 2e-3
+

@@ -356,3 +356,15 @@ def test_layernorm_modulate_pinned(oracle):
     z32 = oracle.np_layernorm_modulate16(x, np.zeros(96, np.float32), None, 1e-6, "f32")
     assert np.array_equal(z32, oracle.np_layernorm_modulate16(x, None, None, 1e-6, "f32"))
     assert not oracle.np_layernorm_modulate16(x, np.zeros(96, np.float16), None, 1e-6, "f16").any()
+    # "affine": the LayerNorm's own weight and bias, no + 1; the fp32 gate of the residual update multiplies in fp32
+    aff = oracle.np_layernorm_modulate16(x, sc32 + 1, sh32, 1e-6, "affine")
+    assert np.array_equal(aff, oracle.np_layernorm_modulate16(x, sc32, sh32, 1e-6, "f32")) or \
+        np.max(np.abs(aff.astype(np.float64) - got32)) <= 2.0 ** -10 * np.maximum(1, np.abs(want32)).max()
+    res = np.array([[1.0, 2.0]], np.float32)
+    y = np.array([[1.0009765625, -3.0]], np.float16)
+    g = np.array([1.0009765625, 0.5], np.float32)
+    # (1 + 2^-10)^2 keeps its 2^-20 term in fp32 (the fp16 gate would round it away)
+    assert np.array_equal(oracle.np_gated_residual32(res, y, g),
+                          np.array([[np.float32(1) + np.float32(1.0009765625) ** 2, 0.5]], np.float32))
+    assert np.array_equal(oracle.np_gated_residual32(res, y), res + y.astype(np.float32))
+
