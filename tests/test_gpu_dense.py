@@ -54,6 +54,10 @@ CASES = [
     (1024, 256, 512, 8, 512),     # q8 with nib == K (many palettes -> global or shared)
     (130, 70, 100, 6, 32),        # K % 32 != 0 -> generic kernel
     (130, 70, 128, 6, 24),        # nib % 32 != 0 -> generic kernel
+    (1024, 200, 512, 6, 4096),    # big tile, ragged N only
+    (1536, 384, 256, 5, 1024),    # q5p, a palette block per four rows
+    (4100, 130, 128, 4, 512),     # ragged last token tile and a two-row last feature tile
+    (2048, 256, 192, 6, 64),      # the palette block changes inside a row every two K-tiles
 ]
 
 
@@ -203,7 +207,8 @@ def test_dense_flux_qkv_full_size_sampled(dthip, oracle, torch_cuda):
         assert float((a.float() * 2 - b.float()).abs().max()) <= 2.0 ** -23
 
 
-@pytest.mark.parametrize("M,head_dim,q,nib", [(700, 128, 6, 4096), (300, 128, 8, 16384), (130, 64, 6, 4096)])
+@pytest.mark.parametrize("M,head_dim,q,nib", [(700, 128, 6, 4096), (300, 128, 8, 16384), (130, 64, 6, 4096),
+                                              (1024, 128, 6, 4096), (4200, 128, 5, 1024)])
 def test_dense_fused_head_norm_rope(dthip, oracle, torch_cuda, M, head_dim, q, nib):
     """x_q / x_k / x_v with the per-head RMSNorm + RoPE of Q and K fused behind the projection (V left plain):
     equals Dense -> RMSNorm(axis: [3]) -> cmul(rot) of the oracle.  head_dim 128 runs inside the GEMM epilogue,
