@@ -1,0 +1,852 @@
+// K1 kernel template and its per-bit-width launcher, shared by dt_dense.hip (host side) and the
+// dt_dense_q*.hip translation units that instantiate it (one per index width, so they build in parallel).
+#pragma once
+#include <numeric>
+
+#include "dt_common.h"
+#include "dt_layout.h"
+#include "dt_qkprep.h"
+
+namespace dt {
+
+constexpr int kMaxWeights = 8;
+constexpr int kMaxGroups = 4;
+constexpr int BK = 32;
+constexpr int kPalLdsBytes = 32768;
+
+enum PalMode : int {
+  kPalShared = 0,  // palettes of every block the tile's rows touch, loaded once, slot = block - first block
+  kPalRow = 1,     // one palette per row in a transposed table, a row's column rewritten where its block changes
+  kPalGlobal = 2,  // lookups go to global memory (any layout)
+  kPlainF16 = 3    // weight is plain fp16, no palette
+};
+
+struct DenseWeight {
+  const uint8_t* data;
+  const uint16_t* bias;
+  uint16_t* y;
+  int64_t ldy;
+  int32_t n;           // rows of this weight
+  int32_t tile_begin;  // first N-tile index of this weight
+  // optional fused epilogue on 128-wide heads: RMSNorm weight, RoPE table, its first row, epsilon
+  const uint16_t* gamma;
+  const uint16_t* rot;
+  int64_t rot_pos0;
+  float eps;
+  // optional elementwise tail: scalar scale, fp16 addend, activation, per-feature gate, accumulation into an
+  // fp32 residual stream
+  float scale;           // 1 = none
+  const uint16_t* add;   // [m, n] fp16 with row stride ld_add; null = none
+  int64_t ld_add;
+  int32_t act;          // DT_ACT_*
+  const uint16_t* gate;  // [n] or null
+  float* res;            // [m, n] fp32 with row stride ld_res, updated in place; null = none
+  int64_t ld_res;
+  const float* gate32;   // [n] fp32 or null: the residual receives float(result) * gate32 (no fp16 product)
+};
+
+// The elementwise tail on one value that has already been rounded to fp16, with
+// the rounding the op-by-op graph applies: after the scale, after the addition,
+// after the activation and after the gate.
+__device__ __forceinline__ float act_gelu_tanh(float x) {
+  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  const float e = __builtin_amdgcn_exp2f(u * 2.885390081777927f);  // exp(2u)
+  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);   // tanh(u)
+  return 0.5f * x * (1.0f + t);
+}
+__device__ __forceinline__ float act_swish(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+__device__ __forceinline__ float post_value(float v, float scale, bool has_add, float add, int act, bool has_gate,
+                                            float gate) {
+  if (scale != 1.0f) v = (float)(half_t)(v * scale);
+  if (has_add) v = (float)(half_t)(v + add);
+  if (act == DT_ACT_GELU_TANH) v = (float)(half_t)act_gelu_tanh(v);
+  else if (act == DT_ACT_SWISH) v = (float)(half_t)act_swish(v);
+  if (has_gate) v = (float)(half_t)(v * gate);
+  return v;
+}
+
+// One X with the weights applied to it; a launch runs up to kMaxGroups of them
+// (same K and weight format), their tiles numbered one group after the other.
+struct DenseGroup {
+  const uint16_t* x;
+  int64_t ldx;
+  int32_t m;
+  int32_t tiles_m, tiles_n;
+  int32_t tile_begin;    // first tile of this group in the launch
+  int32_t w_begin, w_end;  // its weights in DenseArgs::w
+};
+
+struct DenseArgs {
+  int32_t k;
+  int32_t nib;
+  int32_t pal_step;  // K-tiles between columns at which a row can enter a new palette block: gcd(K, nib) / 32
+  int32_t n_groups;
+  int32_t total_tiles;
+  DenseGroup g[kMaxGroups];
+  DenseWeight w[kMaxWeights];
+};
+
+__device__ __forceinline__ uint4_t ld_global_16(const void* p) {
+  return *reinterpret_cast<const uint4_t*>(p);
+}
+
+// Per-thread cursor over one weight row's packed indices, advanced one K-tile
+// (32 elements) at a time so the main loop needs no division.
+struct RowCursor {
+  uint32_t off;   // byte offset of the current granule's first index dword
+  uint32_t poff;  // byte offset of the current block's palette
+  int32_t r;      // element offset inside the current block (multiple of 32)
+  int32_t slot;   // palette slot in LDS (shared mode: block - first block of the tile)
+};
+
+// LDS tiles are [rows][32 halfs] with 64-byte rows and no padding; the 16-byte
+// chunk c of row r lives at chunk c ^ ((r >> 2) & 3).  The LDS of this part
+// serves 16 lanes of a 16-byte access per clock over 64 banks, so 16
+// consecutive rows of one chunk column (the MFMA operand reads and the
+// unpackers' row-per-lane writes) must land on 16 distinct 16-byte bank
+// groups: 4 * (r % 4) + (c ^ (r / 4 % 4)) does.  Measured conflict-free for
+// the operand reads, the 4-lanes-per-row tile writes and the row-per-lane writes.
+__device__ __forceinline__ int lds_chunk(int row, int c) { return row * BK + ((c ^ ((row >> 2) & 3)) << 3); }
+
+// Pair slots are [rows][64 halfs] (two K-tiles side by side): logical chunk c
+// (0..7) of row r sits at 16-byte slot c ^ (r / 2 % 8), which puts 16
+// consecutive rows of one chunk column on 16 distinct 16-byte bank groups.
+__device__ __forceinline__ int pair_chunk(int row, int slot) { return slot ^ ((row >> 1) & 7); }
+
+constexpr int kWaitVm0Lgkm0 = 0x0070;  // s_waitcnt vmcnt(0) lgkmcnt(0)
+constexpr int kWaitLgkm0 = 0xc07f;     // s_waitcnt lgkmcnt(0)
+
+
+__device__ __forceinline__ uint32_t pack_h2(float a, float b) {
+  return (uint32_t)half_to_bits((half_t)a) | ((uint32_t)half_to_bits((half_t)b) << 16);
+}
+
+// 512 threads = 8 waves, two per SIMD, all eight running MFMAs on a (BN/2) x
+// (BM/4) slice.  Every thread issues its share of the memory -> LDS transfer of
+// X and unpacks / looks up half a granule (16 weights) of one W row per
+// K-tile, so the LDS instructions -- the scarce resource: a wave can issue one
+// only every few tens of clocks and the CU's LDS pipe handles one every 2-4 --
+// are spread evenly over all waves and between their MFMAs.  The accumulators
+// are held transposed (rows = output features n, columns = tokens m) so that
+// each lane ends up with runs of consecutive n for one token: 16-byte stores.
+// POST selects the epilogue with the elementwise tail.
+template <int Q, int BM, int BN, int MODE, bool POST>
+__global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
+  constexpr int WN = BN / 2, WM = BM / 4;   // per-wave slice: WN features x WM tokens
+  constexpr int TN = WN / 32, TM = WM / 32;
+  constexpr int AP = BM * (BK / 4) / 512;  // 16-byte chunks of X per thread per pair of K-tiles
+  constexpr int BP = MODE == kPlainF16 ? BN * (BK / 4) / 512 : 0;  // plain fp16 weight: the same
+  constexpr int QW = MODE == kPlainF16 ? 1 : Q;  // dwords per granule
+  constexpr int HW = (QW + 1) / 2;               // dwords that hold either half of a granule
+  constexpr int NST = 3;                         // ring depth of the unpacked weight tiles
+  constexpr int B_STAGE = BN * BK;
+  constexpr int PROW = 2 * BK;                   // halfs per row of a pair slot
+  static_assert(BM % 128 == 0 && BN % 128 == 0 && BN <= 256, "tile");
+
+  // X (and a plain fp16 W) lives in two pair slots, each holding two K-tiles
+  // as [rows][64 halfs]: one is read while the next pair is in flight into the other.
+  __shared__ __attribute__((aligned(1024))) half_t XsA[BM * PROW];
+  __shared__ __attribute__((aligned(1024))) half_t XsB[BM * PROW];
+  __shared__ __attribute__((aligned(1024))) half_t WpA[MODE == kPlainF16 ? BN * PROW : 8];
+  __shared__ __attribute__((aligned(1024))) half_t WpB[MODE == kPlainF16 ? BN * PROW : 8];
+  __shared__ __attribute__((aligned(16))) half_t Bs[MODE == kPlainF16 ? 8 : NST * B_STAGE];
+  // the strictest alignment puts the palettes first in LDS, where their address fits an instruction offset
+  __shared__ __attribute__((aligned(4096))) uint16_t Pal[(MODE == kPalShared || MODE == kPalRow) ? kPalLdsBytes / 2 : 8];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const bool second = wave >= 4;     // unpacks weights 16..31 of its row's granule (waves 0-3: weights 0..15)
+  const int lt = tid & 255;
+  const int wn = wave & 1, wm = (wave >> 1) & 1 | ((wave >> 2) << 1);  // waves w and w+4 share a SIMD and take different m slices
+
+  // Tile order: bands of 8 token tiles; inside a band feature tiles outermost,
+  // token tiles innermost.  Workgroups are dealt round-robin to the 8 XCDs;
+  // giving each XCD a contiguous run of that order makes the workgroups that
+  // run together on an XCD cover a compact 2-D block of tiles (8 x 4 at 32 CUs),
+  // so every X and W panel slice is fetched into that XCD's L2 once per block
+  // instead of once per tile column.
+  const int total = a.total_tiles;
+  int bid = blockIdx.x;
+  {
+    const int per = total / 8;
+    if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
+  }
+  int gi = 0;
+#pragma unroll
+  for (int i = 1; i < kMaxGroups; i++)
+    if (i < a.n_groups && bid >= a.g[i].tile_begin) gi = i;
+  const DenseGroup g = a.g[gi];
+  bid -= g.tile_begin;
+  int tm, tn;
+  {
+    constexpr int GM = 8;
+    const int band_tiles = GM * g.tiles_n;
+    const int band = bid / band_tiles;
+    const int in_band = bid - band * band_tiles;
+    const int rows_in_band = (g.tiles_m - band * GM) < GM ? (g.tiles_m - band * GM) : GM;
+    tn = in_band / rows_in_band;
+    tm = band * GM + (in_band - tn * rows_in_band);
+  }
+
+  int wi = g.w_begin;
+#pragma unroll
+  for (int i = 1; i < kMaxWeights; i++)
+    if (i > g.w_begin && i < g.w_end && tn >= a.w[i].tile_begin) wi = i;
+  const DenseWeight w = a.w[wi];
+  const int n0 = (tn - w.tile_begin) * BN;
+  const int m0 = tm * BM;
+  const int K = a.k;
+  const int nk = K / BK;
+  const QxLayout lay = make_layout(Q, a.nib);
+  const uint32_t pal_bytes = (uint32_t)lay.pal_bytes;
+  // ---- per-thread load coordinates (32-bit byte offsets from uniform bases) ----
+  // X (and a plain fp16 W) goes from memory straight into LDS, two K-tiles at
+  // a time: eight lanes cover one row's 128 contiguous bytes, so every cache
+  // line is requested once, whole.  A wave's load instruction fills 1 KB of
+  // LDS = 8 rows of a pair slot, lane l landing on 16-byte slot l % 8 of row
+  // l / 8; the lane fetches the chunk that the swizzle assigns to that slot.
+  uint32_t a_off[AP];
+#pragma unroll
+  for (int i = 0; i < AP; i++) {
+    const int row = 8 * (wave * AP + i) + (lane >> 3);
+    const int c8 = pair_chunk(row, lane & 7);
+    int gm = m0 + row;
+    if (gm >= g.m) gm = g.m - 1;
+    a_off[i] = (uint32_t)(((int64_t)gm * g.ldx + c8 * 8) * 2);
+  }
+  const char* xbase = reinterpret_cast<const char*>(g.x);
+  const char* wbase = reinterpret_cast<const char*>(w.data);
+
+  // weight row of this thread (two threads per row; each loads and unpacks one half of the row's granule)
+  const int b_row = lt < BN ? lt : BN - 1;
+  RowCursor cur;
+  int64_t pal_first_block = 0;
+  if constexpr (MODE == kPalShared) pal_first_block = ((int64_t)n0 * K) / a.nib;
+  if constexpr (MODE != kPlainF16) {
+    int gn = n0 + b_row;
+    if (gn >= w.n) gn = w.n - 1;
+    const int64_t e = (int64_t)gn * K;
+    const int64_t blk = e / a.nib;
+    const int64_t r = e - blk * a.nib;
+    cur.off = (uint32_t)index_byte_offset(lay, blk, r);
+    cur.poff = (uint32_t)palette_offset(lay, blk);
+    cur.r = (int32_t)r;
+    cur.slot = MODE == kPalShared ? (int32_t)(blk - pal_first_block) : b_row;
+    if (second) cur.off += 4 * (Q / 2);  // first dword that holds an index of the granule's second half
+  }
+  uint32_t bf_off[BP > 0 ? BP : 1];
+  if constexpr (MODE == kPlainF16) {
+#pragma unroll
+    for (int i = 0; i < BP; i++) {
+      const int row = 8 * (wave * BP + i) + (lane >> 3);
+      const int c8 = pair_chunk(row, lane & 7);
+      int gn = n0 + row;
+      if (gn >= w.n) gn = w.n - 1;
+      bf_off[i] = (uint32_t)(((int64_t)gn * K + c8 * 8) * 2);
+    }
+  }
+
+  // ---- palettes -> LDS --------------------------------------------------
+  if constexpr (MODE == kPalShared) {
+    int last_row = n0 + BN - 1;
+    if (last_row >= w.n) last_row = w.n - 1;
+    int64_t last_block = ((int64_t)last_row * K + (K - 1)) / a.nib;
+    int n_pal = (int)(last_block - pal_first_block + 1);
+    const int per_pal = 1 << (Q - 1);  // dwords per palette
+    for (int i = tid; i < n_pal * per_pal; i += 512) {
+      int p = i / per_pal, e = i - p * per_pal;
+      const uint32_t* src =
+          reinterpret_cast<const uint32_t*>(w.data + palette_offset(lay, pal_first_block + p));
+      reinterpret_cast<uint32_t*>(Pal)[i] = src[e];
+    }
+  }
+  // kPalRow: Pal is a table [128-row group][entry][row % 64][row / 64 % 2] of
+  // fp16: rows r and r + 64 share a dword, so the 64 lanes of a wave (64
+  // consecutive rows, one entry each) hit 64 different banks whatever entries
+  // they ask for.  Each of a row's two threads keeps half of the row's column current.
+  const int pal_col = (b_row >> 7) * (256 << Q) + (b_row & 63) * 4 + ((b_row >> 6) & 1) * 2;  // byte offset of this row's column
+  auto fill_pal_column = [&](int64_t blk) {
+    constexpr int ND = (1 << Q) / 4;  // dwords of palette per thread
+    const uint32_t* src =
+        reinterpret_cast<const uint32_t*>(w.data + palette_offset(lay, blk)) + (second ? ND : 0);
+    char* dst = reinterpret_cast<char*>(Pal) + pal_col + (second ? (128 << Q) : 0);
+#pragma unroll
+    for (int d = 0; d < ND; d++) {
+      const uint32_t v = src[d];
+      *reinterpret_cast<uint16_t*>(dst + (2 * d) * 256) = (uint16_t)v;
+      *reinterpret_cast<uint16_t*>(dst + (2 * d + 1) * 256) = (uint16_t)(v >> 16);
+    }
+  };
+  int gn_row = n0 + b_row;  // this thread's weight row
+  if (gn_row >= w.n) gn_row = w.n - 1;
+  // rewrites the column if the row enters a new block at K-tile `tile`
+  auto refresh_pal_column = [&](int tile) {
+    const int64_t e = (int64_t)gn_row * K + (int64_t)tile * BK;
+    const int64_t blk = e / a.nib;
+    if (e == blk * a.nib) fill_pal_column(blk);
+  };
+  int next_pal_tile = a.pal_step;  // next K-tile at which some row may change block
+  if constexpr (MODE == kPalRow) fill_pal_column(((int64_t)gn_row * K) / a.nib);
+
+  // ---- staging --------------------------------------------------------------
+  struct IdxSet {
+    uint32_t b[HW];  // the dwords that hold this thread's half of the row's granule
+    uint32_t poff;
+    int32_t slot;
+  };
+  IdxSet WS[2];  // tile T travels in WS[T % 2]
+  const int last_pair = nk / 2 - 1;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+
+  // Part i (of AP + BP) of the memory -> LDS transfer of K-tile pair q into a
+  // pair slot (pairs past the end re-read the last one, harmlessly).
+  auto issue_pair_part = [&](half_t* xs, half_t* wp, int q, int i) {
+    if (q > last_pair) q = last_pair;
+    const int64_t kb = (int64_t)q * (4 * BK);  // byte offset of the pair inside a row
+    if (i < AP) {
+      load_to_lds_16(xbase + kb, a_off[i], lds_address(xs) + (uint32_t)((wave_u * AP + i) * 1024));
+    } else if constexpr (MODE == kPlainF16) {
+      load_to_lds_16(wbase + kb, bf_off[i - AP], lds_address(wp) + (uint32_t)((wave_u * BP + i - AP) * 1024));
+    }
+  };
+  auto issue_pair = [&](half_t* xs, half_t* wp, int q) {
+#pragma unroll
+    for (int i = 0; i < AP + BP; i++) issue_pair_part(xs, wp, q, i);
+  };
+
+  // Loads the indices of the tile the cursor points at (the last tile is re-read
+  // harmlessly by the final iterations) and moves the cursor on by one tile.
+  int issued = 0;  // tiles loaded so far
+  auto issue_idx = [&](IdxSet& R) {
+    if constexpr (MODE != kPlainF16) {
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(wbase + cur.off);
+#pragma unroll
+      for (int i = 0; i < HW; i++) R.b[i] = src[i];
+      R.poff = cur.poff;
+      R.slot = cur.slot;
+      if (issued + 1 < nk) {
+        issued++;
+        cur.r += BK;
+        cur.off += 4 * Q;
+        if (cur.r >= a.nib) {
+          cur.r = 0;
+          cur.off += pal_bytes;
+          cur.poff += (uint32_t)lay.block_stride;
+          if constexpr (MODE == kPalShared) cur.slot++;
+        }
+      }
+    }
+  };
+
+  // Staging of a weight tile, in pieces that the main loop spreads between its
+  // MFMAs: unpack the 16 indices into palette byte offsets, look them up one
+  // by one, write the 16 weights as two 16-byte chunks.  Threads past the tile's
+  // last row repeat that row's work and write the same bytes again.
+  uint32_t la[16];  // palette byte offsets, then the looked-up weights
+  uint32_t be[HW + 1];
+  const char* gpal = nullptr;
+  uint32_t pal_base = 0;
+  // piece 0 also turns the index dwords into a bit string; piece p yields offsets 4p .. 4p+3
+  auto unpack_piece = [&](IdxSet& R, int p) {
+    if constexpr (MODE != kPlainF16) {
+      if (p == 0) {
+        own_bits<Q, HW>(R.b, second, be);
+        if constexpr (MODE == kPalRow) pal_base = (uint32_t)pal_col;
+        else if constexpr (MODE == kPalGlobal) gpal = wbase + R.poff;
+        else pal_base = (uint32_t)R.slot << (Q + 1);
+      }
+#pragma unroll
+      for (int j = 4 * p; j < 4 * p + 4; j++)
+        la[j] = own_index_at<Q, HW, (MODE == kPalRow ? 8 : 1)>(be, j, pal_base);
+    }
+  };
+  auto lookup = [&](int j) {
+    if constexpr (MODE == kPalGlobal)
+      la[j] = *reinterpret_cast<const uint16_t*>(gpal + la[j]);
+    else if constexpr (MODE != kPlainF16)
+      la[j] = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(Pal) + la[j]);
+  };
+  // Written as assembly, like the transfers: the closing s_waitcnt of an
+  // iteration covers these stores, and the compiler has no reason to order
+  // them against anything else.
+  const uint32_t w_dst = lds_address(Bs) + 2u * (uint32_t)lds_chunk(b_row, second ? 2 : 0);
+  auto write_weights = [&](int stage, int h) {
+    if constexpr (MODE != kPlainF16) {
+      const uint4_t v = {la[8 * h] | (la[8 * h + 1] << 16), la[8 * h + 2] | (la[8 * h + 3] << 16),
+                         la[8 * h + 4] | (la[8 * h + 5] << 16), la[8 * h + 6] | (la[8 * h + 7] << 16)};
+      const uint32_t addr = (w_dst + (uint32_t)(stage * B_STAGE * 2)) ^ (uint32_t)(h << 4);  // chunks c0, c0 + 1 differ in bit 4
+      asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
+    }
+  };
+  auto stage_to_lds = [&](IdxSet& R, int stage) {  // all at once (prologue)
+#pragma unroll
+    for (int p = 0; p < 4; p++) unpack_piece(R, p);
+#pragma unroll
+    for (int j = 0; j < 16; j++) lookup(j);
+    write_weights(stage, 0);
+    write_weights(stage, 1);
+  };
+  // Makes the wait for an index load happen here rather than at its first use.
+  auto touch = [&](IdxSet& R) {
+    if constexpr (MODE != kPlainF16) {
+#pragma unroll
+      for (int j = 0; j < HW; j++) asm volatile("" : "+v"(R.b[j]));
+    }
+  };
+
+  float16_t acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; i++)
+#pragma unroll
+    for (int j = 0; j < TM; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+  // ---- fragment double buffer --------------------------------------------
+  // MFMA A operand = W rows (features), B operand = X rows (tokens); lane holds
+  // row (lane & 31), k-slots 8 * (lane / 32) .. + 7 of the 16-wide k-step.
+  // In a pair slot the 16-byte chunk c (0..7: tile parity * 4 + k-step * 2 +
+  // half) of row r sits at slot c ^ (r / 2 % 8); rows 32 apart share a swizzle.
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int xrow = wm * WM + l32, wrow = wn * WN + l32;
+  const int x_lane = xrow * PROW + ((hi ^ ((xrow >> 1) & 7)) << 3);  // halfs; chunk bits xor'ed per read
+  const int w_lane = wrow * PROW + ((hi ^ ((wrow >> 1) & 7)) << 3);
+  half8_t fw[2][TN], fx[2][TM];
+  // par: tile of the pair (0/1), ks: k-step of the tile, stage: ring stage of the unpacked weights
+  auto read_w = [&](int buf, int i, const half_t* wp, int par, int stage, int ks) {
+    if constexpr (MODE == kPlainF16)
+      fw[buf][i] = *reinterpret_cast<const half8_t*>(wp + (w_lane ^ ((4 * par + 2 * ks) << 3)) + i * 32 * PROW);
+    else
+      fw[buf][i] = *reinterpret_cast<const half8_t*>(Bs + stage * B_STAGE + lds_chunk(wrow + i * 32, 2 * ks + hi));
+  };
+  auto read_x = [&](int buf, int j, const half_t* xs, int par, int ks) {
+    fx[buf][j] = *reinterpret_cast<const half8_t*>(xs + (x_lane ^ ((4 * par + 2 * ks) << 3)) + j * 32 * PROW);
+  };
+  auto mfma = [&](int buf, int i, int j) {
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[buf][i], fx[buf][j], acc[i][j], 0, 0, 0);
+  };
+
+  // ---- prologue: pair 0 in slot A, weights of tiles 0 and 1 in the ring --------
+  issue_pair(XsA, WpA, 0);
+  issue_idx(WS[0]);  // tile 0
+  issue_idx(WS[1]);  // tile 1
+  __syncthreads();   // palettes visible
+  stage_to_lds(WS[0], 0);
+  issue_idx(WS[0]);  // tile 2
+  if constexpr (MODE == kPalRow) {
+    if (next_pal_tile == 1) {  // tile 1 may already start a new palette block
+      __syncthreads();
+      refresh_pal_column(1);
+      next_pal_tile += a.pal_step;
+      __syncthreads();
+    }
+  }
+  stage_to_lds(WS[1], 1);
+  issue_idx(WS[1]);  // tile 3
+  __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < TN; i++) read_w(0, i, WpA, 0, 0, 0);
+#pragma unroll
+  for (int j = 0; j < TM; j++) read_x(0, j, XsA, 0, 0);
+
+  // Iteration t: MFMAs of tile t (pair t / 2) while the weights of tile t+2
+  // are unpacked into ring stage (t+2) % 3.  An even iteration starts the
+  // transfer of the next pair into the other slot (free since the barrier
+  // that ended tile t-1) and waits for it before its closing barrier, because
+  // the odd iteration reads one k-step ahead into that pair.  Index registers
+  // are refilled in odd iterations only, so the even iteration's wait covers
+  // nothing that was issued just before it.
+  //
+  // A wave issues in order, and an LDS instruction occupies it for tens of
+  // clocks, so the iteration is written as 16 slots of one MFMA followed by
+  // a share of the LDS and VALU work: the fragment reads of the next k-step,
+  // the palette lookups and the weight writes all issue while an MFMA of the
+  // same wave (or of the wave it shares the SIMD with) is executing.
+  int s_cur = 0, s_nxt = 1, s_fill = 2;
+  auto iteration = [&](int t, int par, half_t* xs, half_t* wp, half_t* xs_other, half_t* wp_other) {
+    if constexpr (MODE == kPalRow) {
+      if (t + 2 == next_pal_tile) {
+        // lookups of tile t+1 finished before the last barrier
+        if (t + 2 < nk) refresh_pal_column(t + 2);
+        next_pal_tile += a.pal_step;
+        __syncthreads();
+      }
+    }
+    IdxSet& R = WS[par];
+    // the wait for the indices comes here, before the transfer goes out: vector
+    // memory loads return in order, so a wait with the transfer outstanding
+    // would last until it lands
+    touch(R);
+    if (par) issue_idx(WS[0]);  // tile t+3
+    const half_t* xs_n = par == 0 ? xs : xs_other;  // fragments of tile t+1, k-step 0
+    const half_t* wp_n = par == 0 ? wp : wp_other;
+    constexpr int NM = TN * TM;  // MFMAs per k-step = slots per phase
+    constexpr int NF = TN + TM;  // fragment reads per phase
+    constexpr bool packed = MODE != kPlainF16;
+    // Phase 0 (k-step 0): the fragments of k-step 1, one every third place;
+    // between them the parts of the transfer (even iterations), the unpacking,
+    // the refill of the index registers (odd iterations), the first 8 lookups.
+    const int nd = par == 0 ? AP + BP : 0;
+    const int ns0 = nd + (packed ? 4 + par + 8 : 0);
+    auto stage0 = [&](int s) {
+      if (s < nd) { issue_pair_part(xs_other, wp_other, (t >> 1) + 1, s); return; }
+      s -= nd;
+      if (!packed) return;
+      if (s < 4) { unpack_piece(R, s); return; }
+      s -= 4;
+      if (par) {
+        if (s == 0) { issue_idx(WS[1]); return; }  // tile t+4
+        s -= 1;
+      }
+      if (s < 8) lookup(s);
+    };
+    // Phase 1 (k-step 1): the next tile's first fragments (every k-step 0
+    // MFMA has been issued, so their registers are free), the other lookups,
+    // the two weight writes.
+    const int ns1 = packed ? 10 : 0;
+    auto stage1 = [&](int s) {
+      if (!packed) return;
+      if (s < 8) lookup(8 + s);
+      else if (s < 10) write_weights(s_fill, s - 8);
+    };
+    auto read0 = [&](int r) {
+      if (r < TN) read_w(1, r, wp, par, s_cur, 1);
+      else read_x(1, r - TN, xs, par, 1);
+    };
+    auto read1 = [&](int r) {
+      if (r < TN) read_w(0, r, wp_n, par ^ 1, s_nxt, 0);
+      else read_x(0, r - TN, xs_n, par ^ 1, 0);
+    };
+    // place k of a phase: a read at every third place while reads last, stage parts elsewhere
+    auto place = [&](int k, int ns, auto&& rd, auto&& st) {
+      if (k < 3 * NF) {
+        if (k % 3 == 0) rd(k / 3);
+        else if ((k / 3) * 2 + k % 3 - 1 < ns) st((k / 3) * 2 + k % 3 - 1);
+      } else if (k - NF < ns) {
+        st(k - NF);
+      }
+    };
+    const int n0 = NF + (ns0 > 2 * NF ? ns0 : 2 * NF);
+    const int n1 = NF + (ns1 > 2 * NF ? ns1 : 2 * NF);
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+      __builtin_amdgcn_sched_barrier(0);
+      mfma(0, m / TM, m % TM);
+#pragma unroll
+      for (int k = m * n0 / NM; k < (m + 1) * n0 / NM; k++) place(k, ns0, read0, stage0);
+    }
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+      __builtin_amdgcn_sched_barrier(0);
+      mfma(1, m / TM, m % TM);
+#pragma unroll
+      for (int k = m * n1 / NM; k < (m + 1) * n1 / NM; k++) place(k, ns1, read1, stage1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (par == 0)
+      __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+    else
+      __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+    __syncthreads();
+    const int s = s_cur;
+    s_cur = s_nxt;
+    s_nxt = s_fill;
+    s_fill = s;
+  };
+
+  int t = 0;
+  for (; t + 3 < nk; t += 4) {
+    iteration(t, 0, XsA, WpA, XsB, WpB);
+    iteration(t + 1, 1, XsA, WpA, XsB, WpB);
+    iteration(t + 2, 0, XsB, WpB, XsA, WpA);
+    iteration(t + 3, 1, XsB, WpB, XsA, WpA);
+  }
+  if (t < nk) {  // nk is even: two iterations left
+    iteration(t, 0, XsA, WpA, XsB, WpB);
+    iteration(t + 1, 1, XsA, WpA, XsB, WpB);
+  }
+
+  // ---- epilogue with an elementwise tail (activation, gate, fp32 residual) -------
+  // Straight from the accumulators: lane holds token column (lane & 31) and runs
+  // of 4 consecutive features 8 * g + 4 * (lane / 32) + (0..3) per block.
+  if constexpr (POST) {
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      const int gm = m0 + wm * WM + j * 32 + l32;
+      const int64_t gmc = gm < g.m ? gm : 0;
+      uint16_t* yrow = w.y ? w.y + gmc * w.ldy : nullptr;
+      float* rrow = w.res ? w.res + gmc * w.ld_res : nullptr;
+      const uint16_t* arow = w.add ? w.add + gmc * w.ld_add : nullptr;
+      const bool vec = (!w.gate32 || (reinterpret_cast<uintptr_t>(w.gate32) & 15) == 0) &&
+                       (!w.add || (((w.ld_add & 3) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 7) == 0)) &&
+                       (!w.gate || (reinterpret_cast<uintptr_t>(w.gate) & 7) == 0) &&
+                       (!w.bias || (reinterpret_cast<uintptr_t>(w.bias) & 7) == 0) &&
+                       (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0)) &&
+                       (!w.y || (((w.ldy & 3) == 0) && (reinterpret_cast<uintptr_t>(w.y) & 7) == 0));
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int gq = 0; gq < 4; gq++) {
+          const int nn = n0 + wn * WN + i * 32 + 8 * gq + 4 * hi;
+          float bq[4] = {0.f, 0.f, 0.f, 0.f}, gt[4] = {1.f, 1.f, 1.f, 1.f}, rr[4] = {0.f, 0.f, 0.f, 0.f}, pv[4];
+          float ad[4] = {0.f, 0.f, 0.f, 0.f}, g32[4] = {1.f, 1.f, 1.f, 1.f};
+          const bool full = vec && nn + 3 < w.n;
+          if (gm < g.m) {
+            if (full) {
+              if (w.bias) {
+                const uint2_t t2 = *reinterpret_cast<const uint2_t*>(w.bias + nn);
+                bq[0] = (float)bits_to_half((uint16_t)t2[0]); bq[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
+                bq[2] = (float)bits_to_half((uint16_t)t2[1]); bq[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
+              }
+              if (w.gate) {
+                const uint2_t t2 = *reinterpret_cast<const uint2_t*>(w.gate + nn);
+                gt[0] = (float)bits_to_half((uint16_t)t2[0]); gt[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
+                gt[2] = (float)bits_to_half((uint16_t)t2[1]); gt[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
+              }
+              if (w.gate32) {
+                const float4_t t4 = *reinterpret_cast<const float4_t*>(w.gate32 + nn);
+                g32[0] = t4[0]; g32[1] = t4[1]; g32[2] = t4[2]; g32[3] = t4[3];
+              }
+              if (arow) {
+                const uint2_t t2 = *reinterpret_cast<const uint2_t*>(arow + nn);
+                ad[0] = (float)bits_to_half((uint16_t)t2[0]); ad[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
+                ad[2] = (float)bits_to_half((uint16_t)t2[1]); ad[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
+              }
+              if (rrow) {
+                const float4_t t4 = *reinterpret_cast<const float4_t*>(rrow + nn);
+                rr[0] = t4[0]; rr[1] = t4[1]; rr[2] = t4[2]; rr[3] = t4[3];
+              }
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                if (nn + e < w.n) {
+                  if (w.bias) bq[e] = (float)bits_to_half(w.bias[nn + e]);
+                  if (w.gate) gt[e] = (float)bits_to_half(w.gate[nn + e]);
+                  if (rrow) rr[e] = rrow[nn + e];
+                  if (arow) ad[e] = (float)bits_to_half(arow[nn + e]);
+                  if (w.gate32) g32[e] = w.gate32[nn + e];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const float v0 = (float)(half_t)(acc[i][j][4 * gq + e] + bq[e]);
+              pv[e] = post_value(v0, w.scale, arow != nullptr, ad[e], w.act, w.gate != nullptr, gt[e]);
+              float pr = pv[e] * g32[e];  // the product is its own op: rounded before the addition
+              asm volatile("" : "+v"(pr));
+              rr[e] += pr;
+            }
+            if (full) {
+              if (rrow) *reinterpret_cast<float4_t*>(rrow + nn) = float4_t{rr[0], rr[1], rr[2], rr[3]};
+              if (yrow) *reinterpret_cast<uint2_t*>(yrow + nn) = uint2_t{pack_h2(pv[0], pv[1]), pack_h2(pv[2], pv[3])};
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                if (nn + e < w.n) {
+                  if (rrow) rrow[nn + e] = rr[e];
+                  if (yrow) yrow[nn + e] = half_to_bits((half_t)pv[e]);
+                }
+            }
+          }
+        }
+    }
+    return;
+  }
+
+  // ---- fused epilogue: per-head RMSNorm and RoPE on the way out ---------------
+  // A wave's 128 features are exactly one head, and every lane pair (l, l ^ 32)
+  // holds all 128 of them for its token, adjacent (re, im) pairs in one lane:
+  // the norm's reduction and the rotation need no data movement.  Rounds to
+  // fp16 after the Dense, after the norm and after the rotation, as the
+  // op-by-op graph does.
+  if constexpr (WN == 128) {
+    if (w.gamma || w.rot) {
+      const int nh = n0 + wn * WN;  // first feature of this wave's head
+      if (nh >= w.n) return;        // heads are whole: this wave's slice lies past the last one
+#pragma unroll
+      for (int j = 0; j < TM; j++) {
+        const int gm = m0 + wm * WM + j * 32 + l32;
+        const int gmc = gm < g.m ? gm : g.m - 1;
+        uint16_t* yrow = w.y + (int64_t)gmc * w.ldy;
+        float y[TN][16];
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            const int nl = i * 32 + 8 * g + 4 * hi;
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (w.bias) {
+              const uint2_t bb = *reinterpret_cast<const uint2_t*>(w.bias + nh + nl);
+              bv[0] = (float)bits_to_half((uint16_t)bb[0]);
+              bv[1] = (float)bits_to_half((uint16_t)(bb[0] >> 16));
+              bv[2] = (float)bits_to_half((uint16_t)bb[1]);
+              bv[3] = (float)bits_to_half((uint16_t)(bb[1] >> 16));
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const float v = (float)(half_t)(acc[i][j][4 * g + e] + bv[e]);
+              y[i][4 * g + e] = v;
+              ss += v * v;
+            }
+          }
+        if (w.gamma) {
+          const float inv = 1.0f / sqrtf(sum32(ss) / (float)WN + w.eps);
+#pragma unroll
+          for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+              const uint2_t gg = *reinterpret_cast<const uint2_t*>(w.gamma + i * 32 + 8 * g + 4 * hi);
+              const float gv[4] = {(float)bits_to_half((uint16_t)gg[0]), (float)bits_to_half((uint16_t)(gg[0] >> 16)),
+                                   (float)bits_to_half((uint16_t)gg[1]), (float)bits_to_half((uint16_t)(gg[1] >> 16))};
+#pragma unroll
+              for (int e = 0; e < 4; e++) y[i][4 * g + e] = (float)(half_t)(y[i][4 * g + e] * inv * gv[e]);
+            }
+        }
+        if (w.rot) {
+          const uint16_t* rrow = w.rot + (w.rot_pos0 + gmc) * WN;
+#pragma unroll
+          for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+              const uint2_t rr = *reinterpret_cast<const uint2_t*>(rrow + i * 32 + 8 * g + 4 * hi);
+#pragma unroll
+              for (int pr = 0; pr < 2; pr++) {
+                const float c = (float)bits_to_half((uint16_t)rr[pr]), sn = (float)bits_to_half((uint16_t)(rr[pr] >> 16));
+                const float re = y[i][4 * g + 2 * pr], im = y[i][4 * g + 2 * pr + 1];
+                y[i][4 * g + 2 * pr] = (float)(half_t)(re * c - im * sn);
+                y[i][4 * g + 2 * pr + 1] = (float)(half_t)(re * sn + im * c);
+              }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+          uint32_t pk[4][2];
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            pk[g][0] = pack_h2(y[i][4 * g], y[i][4 * g + 1]);
+            pk[g][1] = pack_h2(y[i][4 * g + 2], y[i][4 * g + 3]);
+          }
+#pragma unroll
+          for (int gp = 0; gp < 2; gp++) {
+            uint32_t run[4];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+              auto r = __builtin_amdgcn_permlane32_swap(pk[2 * gp][e], pk[2 * gp + 1][e], false, false);
+              run[e] = r[0];
+              run[2 + e] = r[1];
+            }
+            if (gm < g.m) *reinterpret_cast<uint4_t*>(yrow + nh + i * 32 + 16 * gp + 8 * hi) = uint4_t{run[0], run[1], run[2], run[3]};
+          }
+        }
+      }
+      return;
+    }
+  }
+
+  // ---- epilogue: bias, round once to fp16, 16-byte stores -------------------
+  // Accumulator block (i, j): lane holds token column (lane & 31) and features
+  // 8 * g + 4 * (lane / 32) + (0..3) for g = 0..3.  Swapping the odd groups of
+  // the low half-wave with the even groups of the high half-wave leaves every
+  // lane with runs of 8 consecutive features.
+#pragma unroll
+  for (int j = 0; j < TM; j++) {
+    const int gm = m0 + wm * WM + j * 32 + l32;
+    uint16_t* yrow = w.y + (int64_t)(gm < g.m ? gm : 0) * w.ldy;
+#pragma unroll
+    for (int i = 0; i < TN; i++) {
+      const int nb = n0 + wn * WN + i * 32;
+      uint32_t pk[4][2];
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+        if (w.bias) {
+          const int nn = nb + 8 * g + 4 * hi;
+          if (nn + 3 < w.n) {
+            const uint2_t bb = *reinterpret_cast<const uint2_t*>(w.bias + nn);
+            b0 = (float)bits_to_half((uint16_t)bb[0]);
+            b1 = (float)bits_to_half((uint16_t)(bb[0] >> 16));
+            b2 = (float)bits_to_half((uint16_t)bb[1]);
+            b3 = (float)bits_to_half((uint16_t)(bb[1] >> 16));
+          } else {
+            if (nn < w.n) b0 = (float)bits_to_half(w.bias[nn]);
+            if (nn + 1 < w.n) b1 = (float)bits_to_half(w.bias[nn + 1]);
+            if (nn + 2 < w.n) b2 = (float)bits_to_half(w.bias[nn + 2]);
+          }
+        }
+        pk[g][0] = pack_h2(acc[i][j][4 * g] + b0, acc[i][j][4 * g + 1] + b1);
+        pk[g][1] = pack_h2(acc[i][j][4 * g + 2] + b2, acc[i][j][4 * g + 3] + b3);
+      }
+      // after the swaps: low half-wave holds groups 0 and 2 complete (features
+      // 0..7, 16..23), high half-wave groups 1 and 3 (features 8..15, 24..31)
+#pragma unroll
+      for (int gp = 0; gp < 2; gp++) {
+        uint32_t run[4];
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+          // v_permlane32_swap: first operand's high half <-> second operand's low half
+          auto r = __builtin_amdgcn_permlane32_swap(pk[2 * gp][e], pk[2 * gp + 1][e], false, false);
+          run[e] = r[0];      // low lanes: own group 2gp     | high lanes: low lanes' group 2gp+1
+          run[2 + e] = r[1];  // low lanes: high lanes' 2gp   | high lanes: own group 2gp+1
+        }
+        const int nn = nb + 16 * gp + 8 * hi;
+        if (gm < g.m) {
+          if (nn + 7 < w.n && ((w.ldy & 7) == 0) && ((reinterpret_cast<uintptr_t>(w.y) & 15) == 0)) {
+            *reinterpret_cast<uint4_t*>(yrow + nn) = uint4_t{run[0], run[1], run[2], run[3]};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              if (nn + e < w.n) yrow[nn + e] = (uint16_t)(run[e >> 1] >> (16 * (e & 1)));
+          }
+        }
+      }
+    }
+  }
+}
+
+
+// Tile shapes the host side chooses between.
+enum DenseTile : int { kTile128x128 = 0, kTile128x256 = 1, kTile256x256 = 2 };
+
+template <int Q, int BM, int BN, bool POST>
+static dt_status launch_tiled(hipStream_t s, const DenseArgs& a, int mode) {
+  dim3 grid((unsigned)a.total_tiles), block(512);
+  if constexpr (Q == 16) {  // plain fp16 weight
+    hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, POST>), grid, block, 0, s, a);
+    return launch_status();
+  } else {
+    switch (mode) {
+      case kPalShared: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalShared, POST>), grid, block, 0, s, a); break;
+      case kPalRow:
+        if constexpr ((BN << (Q + 1)) <= kPalLdsBytes) {
+          hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalRow, POST>), grid, block, 0, s, a);
+          break;
+        } else {
+          return DT_NO_KERNEL;  // choose_pal_mode never picks per-row palettes that do not fit
+        }
+      default: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalGlobal, POST>), grid, block, 0, s, a); break;
+    }
+    return launch_status();
+  }
+}
+
+template <int Q, bool POST>
+static dt_status launch_dense_qp(hipStream_t s, const DenseArgs& a, int tile, int mode) {
+  switch (tile) {
+    case kTile128x128: return launch_tiled<Q, 128, 128, POST>(s, a, mode);
+    case kTile128x256: return launch_tiled<Q, 128, 256, POST>(s, a, mode);
+    default: return launch_tiled<Q, 256, 256, POST>(s, a, mode);
+  }
+}
+
+// Every tiled kernel for Q-bit indices (Q = 16: plain fp16 weights); `post` selects the variant with the
+// elementwise tail.  Instantiated once per Q in dt_dense_q<Q>.hip.
+template <int Q>
+dt_status launch_dense_q(hipStream_t s, const DenseArgs& a, int tile, bool post, int mode) {
+  return post ? launch_dense_qp<Q, true>(s, a, tile, mode) : launch_dense_qp<Q, false>(s, a, tile, mode);
+}
+
+}  // namespace dt
