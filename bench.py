@@ -210,6 +210,12 @@ def main():
     ms["dense_plainf16_M4608_N3072"] = time_kernel(
         lambda: pkg.dense_multi(x_all, [wf16], [bias["x_o"]], outs=[y3[0]]), it)
 
+    # the op in front of the block's Dense layers: LayerNorm + adaLN modulation of the fp32 stream (HBM-bound)
+    x32 = torch.randn((S, C), dtype=torch.float32, device=dev)
+    ln_out = torch.empty((S, C), dtype=torch.float16, device=dev)
+    ln_scale, ln_shift = f16((C,), 0.2), f16((C,), 0.2)
+    ms["layernorm_modulate"] = time_kernel(lambda: pkg.layernorm_modulate(x32, ln_scale, ln_shift, 1e-6, out=ln_out), max(it, 10))
+
     tf = lambda flop, t_ms: flop / (t_ms * 1e-3) / 1e12
     kernels = {
         "sdpa_S4608": {"ms": ms["sdpa_S4608"], "tflops": tf(flop_sdpa, ms["sdpa_S4608"]),
@@ -222,6 +228,8 @@ def main():
         "dense_qkv_text+image_one_launch": {"ms": ms["dense_qkv_grouped"], "tflops": tf(2.0 * S * C * 3 * C, ms["dense_qkv_grouped"])},
         "dense_out_text+image_one_launch": {"ms": ms["dense_out_2x"], "tflops": tf(2.0 * S * C * C, ms["dense_out_2x"])},
         "qk_norm_rope": {"ms": ms["qk_norm_rope"], "gbs": 2 * 2 * S * C * 2 / (ms["qk_norm_rope"] * 1e-3) / 1e9},
+        "layernorm_modulate_M4608_C3072": {"ms": ms["layernorm_modulate"], "gbs": 6 * S * C / (ms["layernorm_modulate"] * 1e-3) / 1e9,
+                                           "frac_hbm_peak": 6 * S * C / (ms["layernorm_modulate"] * 1e-3) / 8e12},
     }
     for k in kernels.values():
         if "tflops" in k:
