@@ -17,8 +17,8 @@ from typing import Dict, Optional, Sequence
 
 import numpy as np
 
-from . import (ACT_GELU_TANH, DensePost, HeadEpilogue, QxTensor, dense_grouped, layernorm_modulate, sdpa_segments,
-               _torch)
+from . import (ACT_GELU_TANH, DensePost, HeadEpilogue, QxTensor, dense_grouped, dense_multi, dense_post,
+               layernorm_modulate, sdpa_segments, _torch)
 
 DENSE_NAMES = ("c_q", "c_k", "c_v", "x_q", "x_k", "x_v", "c_o", "x_o", "c_linear1", "c_out_proj", "x_linear1",
                "x_out_proj")
@@ -95,3 +95,47 @@ class JointTransformerBlock:
             dict(x=buf["ch"], weights=[W["c_out_proj"]], biases=[Bv["c_out_proj"]],
                  posts=tail(contextChunks[5], c_res))], stream=stream)
         return c_res.reshape(context.shape), x_res.reshape(x.shape)
+
+
+SINGLE_DENSE_NAMES = ("x_q", "x_k", "x_v", "x_o", "x_linear1", "x_out_proj")
+SINGLE_NORM_NAMES = ("x_norm_q", "x_norm_k")
+
+
+class SingleTransformerBlock:
+    """Flux.1 single-stream block (Models/Flux1.swift:367-492, `contextBlockPreOnly: false`, `.scaleMerged`): one
+    stream of t + hw tokens, attention and feed-forward in parallel on the same modulated input, their fp16 sum gated
+    into the fp32 stream.  Six launches: LayerNorm + modulation; x_q x_k x_v with per-head RMSNorm and RoPE in the
+    epilogue; attention; x_linear1 with GELU(tanh); x_o (no bias); x_out_proj whose epilogue adds the x_o result,
+    applies the gate and accumulates into the residual."""
+
+    def __init__(self, k: int, h: int, tokens: int):
+        self.k, self.h, self.tokens = k, h, tokens
+        self.weight: Dict[str, QxTensor] = {}
+        self.bias: Dict[str, object] = {}
+        self.norm: Dict[str, object] = {}
+
+    def __call__(self, x, rot, xChunks: Sequence[object], stream=None):
+        """x [1, t + hw, h k] fp32, rot [t + hw, k] fp16, xChunks: shift, scale (with its + 1), gate, fp16 [h k].
+        Returns the new x, fp32."""
+        torch = _torch()
+        k, h, S = self.k, self.h, self.tokens
+        C = h * k
+        if tuple(x.shape[-2:]) != (S, C) or len(xChunks) != 3:
+            raise ValueError("x / xChunks do not match the block")
+        W, Bv, G = self.weight, self.bias, self.norm
+        res = x.reshape(S, C).clone()
+        xn = layernorm_modulate(res, xChunks[1], xChunks[0], 1e-6, stream=stream)
+        qkv = torch.empty((S, 3, h, k), dtype=torch.float16, device=x.device)
+        qkv2 = qkv.view(S, 3 * C)
+        dense_multi(xn, [W["x_q"], W["x_k"], W["x_v"]], [Bv["x_q"], Bv["x_k"], Bv["x_v"]],
+                    outs=[qkv2[:, i * C:(i + 1) * C] for i in range(3)], stream=stream,
+                    epilogues=[HeadEpilogue(G["x_norm_q"], rot, 0, 1e-6, k), HeadEpilogue(G["x_norm_k"], rot, 0, 1e-6, k),
+                               None])
+        att = sdpa_segments([qkv[:, 0].unsqueeze(0)], [qkv[:, 1].unsqueeze(0)], [qkv[:, 2].unsqueeze(0)],
+                            1.0 / float(np.sqrt(k)), stream=stream)
+        hid = dense_post(xn, [W["x_linear1"]], [Bv["x_linear1"]], [DensePost(ACT_GELU_TANH)], stream=stream)[0]
+        heads = dense_multi(att.view(S, C), [W["x_o"]], [None], stream=stream)[0]
+        dense_post(hid, [W["x_out_proj"]], [Bv["x_out_proj"]],
+                   [DensePost(gate=xChunks[2], residual=res, keep_output=False, addend=heads)], stream=stream)
+        return res.reshape(x.shape)
+

@@ -470,3 +470,18 @@ def np_wan_attention_block(x32, rot16, chunks32, cK16, cV16, dense, norm, norm3_
     ff = dense["x_out_proj"](np_gelu_tanh16(dense["x_linear1"](xn)))
     return np_gated_residual32(out, ff, chunks32[5])
 
+
+def np_flux_single_block(x32, rot16, xch, dense, norm, k, h):
+    """Flux.1 SingleTransformerBlock op by op (Models/Flux1.swift:367-492; contextBlockPreOnly false): LayerNorm +
+    modulation (:375-376), x_q / x_k / x_v with per-head RMSNorm (:377-386), RoPE (:390-391), attention at
+    1 / sqrt(k) (:431-435), then x_o (no bias) + feed-forward of the same modulated input, summed in fp16, gated and
+    added to the fp32 stream (:452-456).  `dense[name]`: callable X16 -> Y16; `xch`: shift, scale, gate (fp16)."""
+    S = x32.shape[0]
+    xn = np_layernorm_modulate16(x32, xch[1], xch[0], 1e-6, "f16")
+    K_ = C.cmul(C.rmsnorm(dense["x_k"](xn).reshape(S, h, k), norm["x_norm_k"], 1e-6), rot16)
+    Q_ = C.cmul(C.rmsnorm(dense["x_q"](xn).reshape(S, h, k), norm["x_norm_q"], 1e-6), rot16)
+    V_ = dense["x_v"](xn).reshape(S, h, k)
+    att = C.sdpa(Q_[None], K_[None], V_[None], 1.0 / np.sqrt(k))[0].reshape(S, h * k)
+    ff = dense["x_out_proj"](np_gelu_tanh16(dense["x_linear1"](xn)))
+    return np_gated_residual(x32, np_add16(dense["x_o"](att), ff), xch[2])
+

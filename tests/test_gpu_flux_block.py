@@ -105,3 +105,37 @@ def test_wan_attention_block_vs_oracle(dthip, oracle, h, gt, gh, gw, t, q, nib):
     print("x max-abs", mx, "rel-rms", rr, "scale", float(np.abs(want).max()), flush=True)
     assert mx <= 2e-2 and rr <= 2e-3
 
+
+@pytest.mark.parametrize("h,t,gh,gw,q,nib", [(2, 128, 30, 30, 6, 4096), (1, 20, 10, 12, 5, 1024)])
+def test_flux_single_block_vs_oracle(dthip, oracle, h, t, gh, gw, q, nib):
+    """A Flux.1 single-stream block (attention and feed-forward in parallel, summed in fp16, one gate) against the
+    oracle's op-by-op restatement of Models/Flux1.swift:367-492.  Same bar as the joint block."""
+    import torch
+    flux1 = importlib.import_module(dthip.__name__ + ".flux1")
+    k = 128
+    S, C = t + gh * gw, h * k
+    rng = np.random.default_rng(S)
+    blk = flux1.SingleTransformerBlock(k, h, S)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    dense, norm = {}, {}
+    for name in flux1.SINGLE_DENSE_NAMES:
+        N, K = (4 * C, C) if name == "x_linear1" else (C, 4 * C) if name == "x_out_proj" else (C, C)
+        packed, _, _ = oracle.synth_qx_weight(rng, N, K, q, nib, 1.0 / np.sqrt(K))
+        b = None if name == "x_o" else (rng.standard_normal(N) * 0.05).astype(np.float16)
+        blk.weight[name] = dthip.QxTensor.from_packed(packed, q, nib, (N, K))
+        blk.bias[name] = None if b is None else dev(b)
+        dense[name] = (lambda p, n, bb: (lambda X: oracle.C.dense_qx(X, p, q, nib, n, bb)))(packed, N, b)
+    for name in flux1.SINGLE_NORM_NAMES:
+        g = (1 + 0.05 * rng.standard_normal(k)).astype(np.float16)
+        blk.norm[name] = dev(g)
+        norm[name] = g
+    rot = dthip.Flux1RotaryPositionEmbedding(gh, gw, t, channels=k).astype(np.float16)
+    x = (rng.standard_normal((1, S, C)) * 2).astype(np.float32)
+    xch = [(rng.standard_normal(C) * s + o).astype(np.float16) for s, o in ((0.3, 0), (0.2, 1), (0.3, 0))]
+    print("flux single block", h, S, q, nib, flush=True)
+    got = blk(dev(x), dev(rot), [dev(v) for v in xch]).cpu().numpy()[0]
+    want = oracle.np_flux_single_block(x[0], rot, xch, dense, norm, k, h)
+    mx, rr = oracle.err_stats(got, want)
+    print("x max-abs", mx, "rel-rms", rr, "scale", float(np.abs(want).max()), flush=True)
+    assert mx <= 2e-2 and rr <= 2e-3
+
