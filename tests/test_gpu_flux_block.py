@@ -139,3 +139,39 @@ def test_flux_single_block_vs_oracle(dthip, oracle, h, t, gh, gw, q, nib):
     print("x max-abs", mx, "rel-rms", rr, "scale", float(np.abs(want).max()), flush=True)
     assert mx <= 2e-2 and rr <= 2e-3
 
+
+def test_joint_block_replays_as_hip_graph(dthip, oracle):
+    """The twelve launches of a whole joint block (LayerNorm-modulate, grouped Dense with head epilogues and with
+    elementwise tails, attention) captured as one HIP graph: every replay, with eager runs and synchronisations in
+    between, reproduces the eager result bit for bit."""
+    import torch
+    k, h, t, gh, gw = 128, 2, 128, 32, 32
+    hw, C = gh * gw, h * k
+    rng = np.random.default_rng(91)
+    blk, _, _, _ = build_block(dthip, oracle, rng, k, h, t, hw, 6, 4096)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    rot = dev(dthip.Flux1RotaryPositionEmbedding(gh, gw, t, channels=k).astype(np.float16))
+    context = dev(rng.standard_normal((1, t, C)).astype(np.float32))
+    x = dev(rng.standard_normal((1, hw, C)).astype(np.float32))
+    mk = lambda: [dev((rng.standard_normal(C) * 0.3 + o).astype(np.float16)) for o in (0, 1, 0, 0, 1, 0)]
+    cch, xch = mk(), mk()
+    print("joint block as hip graph", flush=True)
+    want_c, want_x = blk(context, x, rot, cch, xch)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        blk(context, x, rot, cch, xch)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got_c, got_x = blk(context, x, rot, cch, xch)
+    for _ in range(3):
+        got_c.zero_(); got_x.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got_c, want_c) and torch.equal(got_x, want_x)
+        again_c, again_x = blk(context, x, rot, cch, xch)  # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(again_c, want_c) and torch.equal(again_x, want_x)
+
