@@ -2,6 +2,7 @@
 // dt_dense_q*.hip translation units that instantiate it (one per index width, so they build in parallel).
 #pragma once
 #include <numeric>
+#include <type_traits>
 
 #include "dt_common.h"
 #include "dt_layout.h"
@@ -49,10 +50,10 @@ struct DenseWeight {
 // the rounding the op-by-op graph applies: after the scale, after the addition,
 // after the activation and after the gate.
 __device__ __forceinline__ float act_gelu_tanh(float x) {
+  // 0.5 x (1 + tanh(u)) = x sigmoid(2u) = x / (1 + exp(-2u)): no cancellation for large negative x
   const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  const float e = __builtin_amdgcn_exp2f(u * 2.885390081777927f);  // exp(2u)
-  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);   // tanh(u)
-  return 0.5f * x * (1.0f + t);
+  const float e = __builtin_amdgcn_exp2f(u * -2.885390081777927f);  // exp(-2u)
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 __device__ __forceinline__ float act_swish(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
@@ -145,15 +146,25 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   constexpr int PROW = 2 * BK;                   // halfs per row of a pair slot
   static_assert(BM % 128 == 0 && BN % 128 == 0 && BN <= 256, "tile");
 
-  // X (and a plain fp16 W) lives in two pair slots, each holding two K-tiles
-  // as [rows][64 halfs]: one is read while the next pair is in flight into the other.
-  __shared__ __attribute__((aligned(1024))) half_t XsA[BM * PROW];
-  __shared__ __attribute__((aligned(1024))) half_t XsB[BM * PROW];
-  __shared__ __attribute__((aligned(1024))) half_t WpA[MODE == kPlainF16 ? BN * PROW : 8];
-  __shared__ __attribute__((aligned(1024))) half_t WpB[MODE == kPlainF16 ? BN * PROW : 8];
-  __shared__ __attribute__((aligned(16))) half_t Bs[MODE == kPlainF16 ? 8 : NST * B_STAGE];
-  // the strictest alignment puts the palettes first in LDS, where their address fits an instruction offset
-  __shared__ __attribute__((aligned(4096))) uint16_t Pal[(MODE == kPalShared || MODE == kPalRow) ? kPalLdsBytes / 2 : 8];
+  // One LDS array, carved up by hand so that the epilogue can reuse all of it.  The palettes come first:
+  // their addresses then fit an instruction offset.  X (and a plain fp16 W) lives in two pair slots, each
+  // holding two K-tiles as [rows][64 halfs]: one is read while the next pair is in flight into the other.
+  constexpr bool HAS_PAL = MODE == kPalShared || MODE == kPalRow;
+  constexpr int PAL_BYTES = HAS_PAL ? kPalLdsBytes : 0;
+  constexpr int XS_BYTES = BM * PROW * 2;
+  constexpr int WP_BYTES = MODE == kPlainF16 ? BN * PROW * 2 : 0;
+  constexpr int BS_BYTES = MODE == kPlainF16 ? 0 : NST * B_STAGE * 2;
+  constexpr int OFF_XA = PAL_BYTES, OFF_XB = OFF_XA + XS_BYTES, OFF_WA = OFF_XB + XS_BYTES, OFF_WB = OFF_WA + WP_BYTES;
+  constexpr int OFF_BS = OFF_WB + WP_BYTES, LOOP_BYTES = OFF_BS + BS_BYTES;
+  constexpr int OUT_BYTES = BM * BN * 2;  // the fp16 output tile, parked here by the epilogue
+  constexpr int LDS_BYTES = LOOP_BYTES > OUT_BYTES ? LOOP_BYTES : OUT_BYTES;
+  __shared__ __attribute__((aligned(4096))) unsigned char smem[LDS_BYTES];
+  half_t* const XsA = reinterpret_cast<half_t*>(smem + OFF_XA);
+  half_t* const XsB = reinterpret_cast<half_t*>(smem + OFF_XB);
+  half_t* const WpA = reinterpret_cast<half_t*>(smem + OFF_WA);
+  half_t* const WpB = reinterpret_cast<half_t*>(smem + OFF_WB);
+  half_t* const Bs = reinterpret_cast<half_t*>(smem + OFF_BS);
+  uint16_t* const Pal = reinterpret_cast<uint16_t*>(smem);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -570,89 +581,166 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     iteration(t + 1, 1, XsA, WpA, XsB, WpB);
   }
 
-  // ---- epilogue with an elementwise tail (activation, gate, fp32 residual) -------
-  // Straight from the accumulators: lane holds token column (lane & 31) and runs
-  // of 4 consecutive features 8 * g + 4 * (lane / 32) + (0..3) per block.
+  if constexpr (POST) {
+  // ---- epilogue --------------------------------------------------------------
+  // The K loop ended with a barrier, so its LDS tiles are free.  Every wave parks
+  // its WN x WM slice -- bias added, rounded to fp16: the Dense's own result -- in
+  // its own part of LDS as [token][feature] rows and then walks it row by row in a
+  // short loop: RPI token rows per trip, CH lanes of 8 consecutive features per
+  // row, so that every access to memory is a whole 16-byte chunk of a row (32 bytes
+  // for the fp32 stream) and the code stays small (a fully unrolled walk over the
+  // accumulators spends most of its time fetching instructions: measured 47 us per
+  // workgroup for the GELU tail, against 7 us for this form).  The tail -- scale,
+  // addend, activation, gate, residual -- runs in that loop, rounding to fp16
+  // wherever the separate ops would.  The plain and head epilogues further down
+  // stay unrolled: they are short enough, and 2-3 % faster that way.
+  constexpr int CH = WN / 8;    // 16-byte chunks per parked row
+  constexpr int RPI = 64 / CH;  // token rows per trip
+  half_t* const park = reinterpret_cast<half_t*>(smem) + wave * (WM * WN);
+  {
+    // Accumulator block (i, j): lane holds token (lane & 31) of the block and
+    // features 8 g + 4 (lane / 32) + (0..3), g = 0..3.  Chunk c of token t is
+    // parked at chunk c ^ (t % CH): the 8-byte writes of 32 tokens spread over the banks.
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+      for (int gq = 0; gq < 4; gq++) {
+        const int nn = n0 + wn * WN + i * 32 + 8 * gq + 4 * hi;
+        float b4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (w.bias) {
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            if (nn + e < w.n) b4[e] = (float)bits_to_half(w.bias[nn + e]);
+        }
+#pragma unroll
+        for (int j = 0; j < TM; j++) {
+          const int t = j * 32 + l32;
+          const uint2_t pk = {pack_h2(acc[i][j][4 * gq] + b4[0], acc[i][j][4 * gq + 1] + b4[1]),
+                              pack_h2(acc[i][j][4 * gq + 2] + b4[2], acc[i][j][4 * gq + 3] + b4[3])};
+          *reinterpret_cast<uint2_t*>(park + t * WN + (((i * 4 + gq) ^ (t & (CH - 1))) << 3) + 4 * hi) = pk;
+        }
+      }
+  }
+  // a wave's LDS operations execute in order: its reads below see the writes above
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  const int c = lane & (CH - 1), rsub = lane / CH;
+  const int nw = n0 + wn * WN;  // first feature of this wave's slice
+  const int nn = nw + 8 * c;    // first of this lane's 8 features
+  if (nw >= w.n) return;
+  // this lane's column data
+  float gt[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) gt[e] = 1.f;
   if constexpr (POST) {
 #pragma unroll
-    for (int j = 0; j < TM; j++) {
-      const int gm = m0 + wm * WM + j * 32 + l32;
-      const int64_t gmc = gm < g.m ? gm : 0;
-      uint16_t* yrow = w.y ? w.y + gmc * w.ldy : nullptr;
-      float* rrow = w.res ? w.res + gmc * w.ld_res : nullptr;
-      const uint16_t* arow = w.add ? w.add + gmc * w.ld_add : nullptr;
-      const bool vec = (!w.gate32 || (reinterpret_cast<uintptr_t>(w.gate32) & 15) == 0) &&
-                       (!w.add || (((w.ld_add & 3) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 7) == 0)) &&
-                       (!w.gate || (reinterpret_cast<uintptr_t>(w.gate) & 7) == 0) &&
-                       (!w.bias || (reinterpret_cast<uintptr_t>(w.bias) & 7) == 0) &&
-                       (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0)) &&
-                       (!w.y || (((w.ldy & 3) == 0) && (reinterpret_cast<uintptr_t>(w.y) & 7) == 0));
+    for (int e = 0; e < 8; e++)
+      if (nn + e < w.n) {
+        if (w.gate) gt[e] = (float)bits_to_half(w.gate[nn + e]);
+        if (w.gate32) gt[e] = w.gate32[nn + e];
+      }
+  }
+  auto lo16 = [](uint32_t v) { return (float)bits_to_half((uint16_t)v); };
+  auto hi16 = [](uint32_t v) { return (float)bits_to_half((uint16_t)(v >> 16)); };
+  // what a row needs from memory before its arithmetic
+  struct RowIn {
+    uint4_t add;
+    float4_t r0, r1;
+  };
+  // FAST: the wave's slice lies inside the matrix and every row meets the vector alignment
+  auto walk = [&](auto fast_tag) {
+    constexpr bool FAST = decltype(fast_tag)::value;
+    auto fetch = [&](int it, RowIn& in) {
+      const int t = it * RPI + rsub;
+      const int64_t gm = m0 + wm * WM + t;
+      if constexpr (POST) {
+        if (w.add) in.add = *reinterpret_cast<const uint4_t*>(w.add + gm * w.ld_add + nn);
+        if (w.res) {
+          in.r0 = *reinterpret_cast<const float4_t*>(w.res + gm * w.ld_res + nn);
+          in.r1 = *reinterpret_cast<const float4_t*>(w.res + gm * w.ld_res + nn + 4);
+        }
+      }
+    };
+    RowIn cur;
+    if constexpr (FAST) fetch(0, cur);
+    for (int it = 0; it < WM / RPI; it++) {
+      const int t = it * RPI + rsub;
+      const int64_t gm = m0 + wm * WM + t;
+      const bool row_ok = FAST || gm < g.m;
+      const int64_t gmc = row_ok ? gm : 0;
+      RowIn nxt;
+      if constexpr (FAST) {
+        if (it + 1 < WM / RPI) fetch(it + 1, nxt);  // before this row's stores: a load behind a store waits for it
+      }
+      const uint4_t raw = *reinterpret_cast<const uint4_t*>(park + t * WN + ((c ^ (t & (CH - 1))) << 3));
+      float v[8] = {lo16(raw[0]), hi16(raw[0]), lo16(raw[1]), hi16(raw[1]),
+                    lo16(raw[2]), hi16(raw[2]), lo16(raw[3]), hi16(raw[3])};
+      float res[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if constexpr (POST) {
+        float ad[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (w.add) {
+          if constexpr (FAST) {
 #pragma unroll
-      for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int gq = 0; gq < 4; gq++) {
-          const int nn = n0 + wn * WN + i * 32 + 8 * gq + 4 * hi;
-          float bq[4] = {0.f, 0.f, 0.f, 0.f}, gt[4] = {1.f, 1.f, 1.f, 1.f}, rr[4] = {0.f, 0.f, 0.f, 0.f}, pv[4];
-          float ad[4] = {0.f, 0.f, 0.f, 0.f}, g32[4] = {1.f, 1.f, 1.f, 1.f};
-          const bool full = vec && nn + 3 < w.n;
-          if (gm < g.m) {
-            if (full) {
-              if (w.bias) {
-                const uint2_t t2 = *reinterpret_cast<const uint2_t*>(w.bias + nn);
-                bq[0] = (float)bits_to_half((uint16_t)t2[0]); bq[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
-                bq[2] = (float)bits_to_half((uint16_t)t2[1]); bq[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
-              }
-              if (w.gate) {
-                const uint2_t t2 = *reinterpret_cast<const uint2_t*>(w.gate + nn);
-                gt[0] = (float)bits_to_half((uint16_t)t2[0]); gt[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
-                gt[2] = (float)bits_to_half((uint16_t)t2[1]); gt[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
-              }
-              if (w.gate32) {
-                const float4_t t4 = *reinterpret_cast<const float4_t*>(w.gate32 + nn);
-                g32[0] = t4[0]; g32[1] = t4[1]; g32[2] = t4[2]; g32[3] = t4[3];
-              }
-              if (arow) {
-                const uint2_t t2 = *reinterpret_cast<const uint2_t*>(arow + nn);
-                ad[0] = (float)bits_to_half((uint16_t)t2[0]); ad[1] = (float)bits_to_half((uint16_t)(t2[0] >> 16));
-                ad[2] = (float)bits_to_half((uint16_t)t2[1]); ad[3] = (float)bits_to_half((uint16_t)(t2[1] >> 16));
-              }
-              if (rrow) {
-                const float4_t t4 = *reinterpret_cast<const float4_t*>(rrow + nn);
-                rr[0] = t4[0]; rr[1] = t4[1]; rr[2] = t4[2]; rr[3] = t4[3];
-              }
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; e++)
-                if (nn + e < w.n) {
-                  if (w.bias) bq[e] = (float)bits_to_half(w.bias[nn + e]);
-                  if (w.gate) gt[e] = (float)bits_to_half(w.gate[nn + e]);
-                  if (rrow) rr[e] = rrow[nn + e];
-                  if (arow) ad[e] = (float)bits_to_half(arow[nn + e]);
-                  if (w.gate32) g32[e] = w.gate32[nn + e];
-                }
+            for (int q = 0; q < 4; q++) {
+              ad[2 * q] = lo16(cur.add[q]);
+              ad[2 * q + 1] = hi16(cur.add[q]);
             }
+          } else if (row_ok) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-              const float v0 = (float)(half_t)(acc[i][j][4 * gq + e] + bq[e]);
-              pv[e] = post_value(v0, w.scale, arow != nullptr, ad[e], w.act, w.gate != nullptr, gt[e]);
-              float pr = pv[e] * g32[e];  // the product is its own op: rounded before the addition
-              asm volatile("" : "+v"(pr));
-              rr[e] += pr;
-            }
-            if (full) {
-              if (rrow) *reinterpret_cast<float4_t*>(rrow + nn) = float4_t{rr[0], rr[1], rr[2], rr[3]};
-              if (yrow) *reinterpret_cast<uint2_t*>(yrow + nn) = uint2_t{pack_h2(pv[0], pv[1]), pack_h2(pv[2], pv[3])};
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; e++)
-                if (nn + e < w.n) {
-                  if (rrow) rrow[nn + e] = rr[e];
-                  if (yrow) yrow[nn + e] = half_to_bits((half_t)pv[e]);
-                }
-            }
+            for (int e = 0; e < 8; e++)
+              if (nn + e < w.n) ad[e] = (float)bits_to_half(w.add[gmc * w.ld_add + nn + e]);
           }
         }
+        if (w.res) {
+          if constexpr (FAST) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              res[e] = cur.r0[e];
+              res[4 + e] = cur.r1[e];
+            }
+          } else if (row_ok) {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              if (nn + e < w.n) res[e] = w.res[gmc * w.ld_res + nn + e];
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          v[e] = post_value(v[e], w.scale, w.add != nullptr, ad[e], w.act, w.gate != nullptr, gt[e]);
+          float pr = w.gate32 ? v[e] * gt[e] : v[e];  // the fp32 gate's product is its own op: rounded before the addition
+          asm volatile("" : "+v"(pr));
+          res[e] += pr;
+        }
+      }
+      const uint4_t out = {pack_h2(v[0], v[1]), pack_h2(v[2], v[3]), pack_h2(v[4], v[5]), pack_h2(v[6], v[7])};
+      if constexpr (FAST) {
+        if constexpr (POST) {
+          if (w.res) {
+            *reinterpret_cast<float4_t*>(w.res + gm * w.ld_res + nn) = float4_t{res[0], res[1], res[2], res[3]};
+            *reinterpret_cast<float4_t*>(w.res + gm * w.ld_res + nn + 4) = float4_t{res[4], res[5], res[6], res[7]};
+          }
+        }
+        if (w.y) *reinterpret_cast<uint4_t*>(w.y + gm * w.ldy + nn) = out;
+      } else if (row_ok) {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          if (nn + e < w.n) {
+            if constexpr (POST) {
+              if (w.res) w.res[gmc * w.ld_res + nn + e] = res[e];
+            }
+            if (w.y) w.y[gmc * w.ldy + nn + e] = (uint16_t)(out[e >> 1] >> (16 * (e & 1)));
+          }
+      }
+      if constexpr (FAST) cur = nxt;
     }
+  };
+  const bool aligned16 = (!w.y || (((w.ldy & 7) == 0) && (reinterpret_cast<uintptr_t>(w.y) & 15) == 0)) &&
+                         (!POST || ((!w.add || (((w.ld_add & 7) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 15) == 0)) &&
+                                    (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0))));
+  if (aligned16 && nw + WN <= w.n && m0 + wm * WM + WM <= g.m) walk(std::true_type{});
+  else walk(std::false_type{});
     return;
   }
 
