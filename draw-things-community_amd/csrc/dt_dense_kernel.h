@@ -120,6 +120,18 @@ constexpr int kWaitVm0Lgkm0 = 0x0070;  // s_waitcnt vmcnt(0) lgkmcnt(0)
 constexpr int kWaitLgkm0 = 0xc07f;     // s_waitcnt lgkmcnt(0)
 
 
+// Sum over the 16 lanes of a DPP row (lanes 16 k .. 16 k + 15), left in every lane of the row.
+__device__ __forceinline__ float row16_sum(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, false));
+  };
+  v += dpp(v, std::integral_constant<int, 0xB1>{});   // quad_perm [1, 0, 3, 2]
+  v += dpp(v, std::integral_constant<int, 0x4E>{});   // quad_perm [2, 3, 0, 1]
+  v += dpp(v, std::integral_constant<int, 0x124>{});  // row_ror 4
+  v += dpp(v, std::integral_constant<int, 0x128>{});  // row_ror 8
+  return v;
+}
+
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
   return (uint32_t)half_to_bits((half_t)a) | ((uint32_t)half_to_bits((half_t)b) << 16);
 }
@@ -581,7 +593,8 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     iteration(t + 1, 1, XsA, WpA, XsB, WpB);
   }
 
-  if constexpr (POST) {
+  const bool head = WN == 128 && !POST && (w.gamma || w.rot);
+  if (POST || head) {
   // ---- epilogue --------------------------------------------------------------
   // The K loop ended with a barrier, so its LDS tiles are free.  Every wave parks
   // its WN x WM slice -- bias added, rounded to fp16: the Dense's own result -- in
@@ -590,10 +603,10 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // row, so that every access to memory is a whole 16-byte chunk of a row (32 bytes
   // for the fp32 stream) and the code stays small (a fully unrolled walk over the
   // accumulators spends most of its time fetching instructions: measured 47 us per
-  // workgroup for the GELU tail, against 7 us for this form).  The tail -- scale,
-  // addend, activation, gate, residual -- runs in that loop, rounding to fp16
-  // wherever the separate ops would.  The plain and head epilogues further down
-  // stay unrolled: they are short enough, and 2-3 % faster that way.
+  // workgroup for the GELU tail, against 7 us for this form).  The tails -- per-head
+  // RMSNorm + RoPE, or scale / addend / activation / gate / residual -- run in that
+  // loop, rounding to fp16 wherever the separate ops would.  The plain epilogue
+  // further down stays unrolled: it is short enough, and 2-3 % faster that way.
   constexpr int CH = WN / 8;    // 16-byte chunks per parked row
   constexpr int RPI = 64 / CH;  // token rows per trip
   half_t* const park = reinterpret_cast<half_t*>(smem) + wave * (WM * WN);
@@ -608,9 +621,17 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         const int nn = n0 + wn * WN + i * 32 + 8 * gq + 4 * hi;
         float b4[4] = {0.f, 0.f, 0.f, 0.f};
         if (w.bias) {
+          if (nn + 3 < w.n && (reinterpret_cast<uintptr_t>(w.bias) & 7) == 0) {
+            const uint2_t bb = *reinterpret_cast<const uint2_t*>(w.bias + nn);
+            b4[0] = (float)bits_to_half((uint16_t)bb[0]);
+            b4[1] = (float)bits_to_half((uint16_t)(bb[0] >> 16));
+            b4[2] = (float)bits_to_half((uint16_t)bb[1]);
+            b4[3] = (float)bits_to_half((uint16_t)(bb[1] >> 16));
+          } else {
 #pragma unroll
-          for (int e = 0; e < 4; e++)
-            if (nn + e < w.n) b4[e] = (float)bits_to_half(w.bias[nn + e]);
+            for (int e = 0; e < 4; e++)
+              if (nn + e < w.n) b4[e] = (float)bits_to_half(w.bias[nn + e]);
+          }
         }
 #pragma unroll
         for (int j = 0; j < TM; j++) {
@@ -631,9 +652,24 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const int nn = nw + 8 * c;    // first of this lane's 8 features
   if (nw >= w.n) return;
   // this lane's column data
-  float gt[8];
+  float gt[8];  // the gate, or the RMSNorm weight of a head tile
 #pragma unroll
   for (int e = 0; e < 8; e++) gt[e] = 1.f;
+  auto lo16 = [](uint32_t v) { return (float)bits_to_half((uint16_t)v); };
+  auto hi16 = [](uint32_t v) { return (float)bits_to_half((uint16_t)(v >> 16)); };
+  if (head && w.gamma) {
+    if ((reinterpret_cast<uintptr_t>(w.gamma) & 15) == 0) {
+      const uint4_t gg = *reinterpret_cast<const uint4_t*>(w.gamma + 8 * c);
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        gt[2 * q] = lo16(gg[q]);
+        gt[2 * q + 1] = hi16(gg[q]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) gt[e] = (float)bits_to_half(w.gamma[8 * c + e]);
+    }
+  }
   if constexpr (POST) {
 #pragma unroll
     for (int e = 0; e < 8; e++)
@@ -642,11 +678,9 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         if (w.gate32) gt[e] = w.gate32[nn + e];
       }
   }
-  auto lo16 = [](uint32_t v) { return (float)bits_to_half((uint16_t)v); };
-  auto hi16 = [](uint32_t v) { return (float)bits_to_half((uint16_t)(v >> 16)); };
   // what a row needs from memory before its arithmetic
   struct RowIn {
-    uint4_t add;
+    uint4_t add;  // the addend, or the RoPE table row of a head tile
     float4_t r0, r1;
   };
   // FAST: the wave's slice lies inside the matrix and every row meets the vector alignment
@@ -655,6 +689,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     auto fetch = [&](int it, RowIn& in) {
       const int t = it * RPI + rsub;
       const int64_t gm = m0 + wm * WM + t;
+      if (head && w.rot) in.add = *reinterpret_cast<const uint4_t*>(w.rot + (w.rot_pos0 + gm) * WN + 8 * c);
       if constexpr (POST) {
         if (w.add) in.add = *reinterpret_cast<const uint4_t*>(w.add + gm * w.ld_add + nn);
         if (w.res) {
@@ -678,6 +713,35 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       float v[8] = {lo16(raw[0]), hi16(raw[0]), lo16(raw[1]), hi16(raw[1]),
                     lo16(raw[2]), hi16(raw[2]), lo16(raw[3]), hi16(raw[3])};
       float res[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (head) {
+        // per-head RMSNorm and RoPE: a parked row is one head, spread over the CH = 16 lanes of a DPP row
+        if (w.gamma) {
+          float ss = 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; e++) ss += v[e] * v[e];
+          ss = row16_sum(ss);
+          const float inv = 1.0f / sqrtf(ss / (float)WN + w.eps);
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = (float)(half_t)(v[e] * inv * gt[e]);
+        }
+        if (w.rot) {
+          uint4_t rr;
+          if constexpr (FAST) {
+            rr = cur.add;
+          } else {
+            const uint16_t* rrow = w.rot + (w.rot_pos0 + gmc) * WN + 8 * c;
+#pragma unroll
+            for (int q = 0; q < 4; q++) rr[q] = (uint32_t)rrow[2 * q] | ((uint32_t)rrow[2 * q + 1] << 16);
+          }
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const float cs = lo16(rr[q]), sn = hi16(rr[q]);
+            const float re = v[2 * q], im = v[2 * q + 1];
+            v[2 * q] = (float)(half_t)(re * cs - im * sn);
+            v[2 * q + 1] = (float)(half_t)(re * sn + im * cs);
+          }
+        }
+      }
       if constexpr (POST) {
         float ad[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         if (w.add) {
@@ -737,102 +801,12 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     }
   };
   const bool aligned16 = (!w.y || (((w.ldy & 7) == 0) && (reinterpret_cast<uintptr_t>(w.y) & 15) == 0)) &&
+                         (!(head && w.rot) || (reinterpret_cast<uintptr_t>(w.rot) & 15) == 0) &&
                          (!POST || ((!w.add || (((w.ld_add & 7) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 15) == 0)) &&
                                     (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0))));
   if (aligned16 && nw + WN <= w.n && m0 + wm * WM + WM <= g.m) walk(std::true_type{});
   else walk(std::false_type{});
     return;
-  }
-
-  // ---- fused epilogue: per-head RMSNorm and RoPE on the way out ---------------
-  // A wave's 128 features are exactly one head, and every lane pair (l, l ^ 32)
-  // holds all 128 of them for its token, adjacent (re, im) pairs in one lane:
-  // the norm's reduction and the rotation need no data movement.  Rounds to
-  // fp16 after the Dense, after the norm and after the rotation, as the
-  // op-by-op graph does.
-  if constexpr (WN == 128) {
-    if (w.gamma || w.rot) {
-      const int nh = n0 + wn * WN;  // first feature of this wave's head
-      if (nh >= w.n) return;        // heads are whole: this wave's slice lies past the last one
-#pragma unroll
-      for (int j = 0; j < TM; j++) {
-        const int gm = m0 + wm * WM + j * 32 + l32;
-        const int gmc = gm < g.m ? gm : g.m - 1;
-        uint16_t* yrow = w.y + (int64_t)gmc * w.ldy;
-        float y[TN][16];
-        float ss = 0.f;
-#pragma unroll
-        for (int i = 0; i < TN; i++)
-#pragma unroll
-          for (int g = 0; g < 4; g++) {
-            const int nl = i * 32 + 8 * g + 4 * hi;
-            float bv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (w.bias) {
-              const uint2_t bb = *reinterpret_cast<const uint2_t*>(w.bias + nh + nl);
-              bv[0] = (float)bits_to_half((uint16_t)bb[0]);
-              bv[1] = (float)bits_to_half((uint16_t)(bb[0] >> 16));
-              bv[2] = (float)bits_to_half((uint16_t)bb[1]);
-              bv[3] = (float)bits_to_half((uint16_t)(bb[1] >> 16));
-            }
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              const float v = (float)(half_t)(acc[i][j][4 * g + e] + bv[e]);
-              y[i][4 * g + e] = v;
-              ss += v * v;
-            }
-          }
-        if (w.gamma) {
-          const float inv = 1.0f / sqrtf(sum32(ss) / (float)WN + w.eps);
-#pragma unroll
-          for (int i = 0; i < TN; i++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-              const uint2_t gg = *reinterpret_cast<const uint2_t*>(w.gamma + i * 32 + 8 * g + 4 * hi);
-              const float gv[4] = {(float)bits_to_half((uint16_t)gg[0]), (float)bits_to_half((uint16_t)(gg[0] >> 16)),
-                                   (float)bits_to_half((uint16_t)gg[1]), (float)bits_to_half((uint16_t)(gg[1] >> 16))};
-#pragma unroll
-              for (int e = 0; e < 4; e++) y[i][4 * g + e] = (float)(half_t)(y[i][4 * g + e] * inv * gv[e]);
-            }
-        }
-        if (w.rot) {
-          const uint16_t* rrow = w.rot + (w.rot_pos0 + gmc) * WN;
-#pragma unroll
-          for (int i = 0; i < TN; i++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-              const uint2_t rr = *reinterpret_cast<const uint2_t*>(rrow + i * 32 + 8 * g + 4 * hi);
-#pragma unroll
-              for (int pr = 0; pr < 2; pr++) {
-                const float c = (float)bits_to_half((uint16_t)rr[pr]), sn = (float)bits_to_half((uint16_t)(rr[pr] >> 16));
-                const float re = y[i][4 * g + 2 * pr], im = y[i][4 * g + 2 * pr + 1];
-                y[i][4 * g + 2 * pr] = (float)(half_t)(re * c - im * sn);
-                y[i][4 * g + 2 * pr + 1] = (float)(half_t)(re * sn + im * c);
-              }
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < TN; i++) {
-          uint32_t pk[4][2];
-#pragma unroll
-          for (int g = 0; g < 4; g++) {
-            pk[g][0] = pack_h2(y[i][4 * g], y[i][4 * g + 1]);
-            pk[g][1] = pack_h2(y[i][4 * g + 2], y[i][4 * g + 3]);
-          }
-#pragma unroll
-          for (int gp = 0; gp < 2; gp++) {
-            uint32_t run[4];
-#pragma unroll
-            for (int e = 0; e < 2; e++) {
-              auto r = __builtin_amdgcn_permlane32_swap(pk[2 * gp][e], pk[2 * gp + 1][e], false, false);
-              run[e] = r[0];
-              run[2 + e] = r[1];
-            }
-            if (gm < g.m) *reinterpret_cast<uint4_t*>(yrow + nh + i * 32 + 16 * gp + 8 * hi) = uint4_t{run[0], run[1], run[2], run[3]};
-          }
-        }
-      }
-      return;
-    }
   }
 
   // ---- epilogue: bias, round once to fp16, 16-byte stores -------------------
