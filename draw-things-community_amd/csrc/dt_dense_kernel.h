@@ -183,7 +183,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const int wave = tid >> 6;
   const bool second = wave >= 4;     // unpacks weights 16..31 of its row's granule (waves 0-3: weights 0..15)
   const int lt = tid & 255;
-  const int wn = wave & 1, wm = (wave >> 1) & 1 | ((wave >> 2) << 1);  // waves w and w+4 share a SIMD and take different m slices
+  const int wn = wave & 1, wm = ((wave >> 1) & 1) | ((wave >> 2) << 1);  // waves w and w+4 share a SIMD and take different m slices
 
   // Tile order: bands of 8 token tiles; inside a band feature tiles outermost,
   // token tiles innermost.  Workgroups are dealt round-robin to the 8 XCDs;
