@@ -594,7 +594,6 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   }
 
   const bool head = WN == 128 && !POST && (w.gamma || w.rot);
-  if (POST || head) {
   // ---- epilogue --------------------------------------------------------------
   // The K loop ended with a barrier, so its LDS tiles are free.  Every wave parks
   // its WN x WM slice -- bias added, rounded to fp16: the Dense's own result -- in
@@ -605,8 +604,8 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // accumulators spends most of its time fetching instructions: measured 47 us per
   // workgroup for the GELU tail, against 7 us for this form).  The tails -- per-head
   // RMSNorm + RoPE, or scale / addend / activation / gate / residual -- run in that
-  // loop, rounding to fp16 wherever the separate ops would.  The plain epilogue
-  // further down stays unrolled: it is short enough, and 2-3 % faster that way.
+  // loop, rounding to fp16 wherever the separate ops would; a plain Dense just
+  // stores the parked rows.
   constexpr int CH = WN / 8;    // 16-byte chunks per parked row
   constexpr int RPI = 64 / CH;  // token rows per trip
   half_t* const park = reinterpret_cast<half_t*>(smem) + wave * (WM * WN);
@@ -806,67 +805,6 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
                                     (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0))));
   if (aligned16 && nw + WN <= w.n && m0 + wm * WM + WM <= g.m) walk(std::true_type{});
   else walk(std::false_type{});
-    return;
-  }
-
-  // ---- epilogue: bias, round once to fp16, 16-byte stores -------------------
-  // Accumulator block (i, j): lane holds token column (lane & 31) and features
-  // 8 * g + 4 * (lane / 32) + (0..3) for g = 0..3.  Swapping the odd groups of
-  // the low half-wave with the even groups of the high half-wave leaves every
-  // lane with runs of 8 consecutive features.
-#pragma unroll
-  for (int j = 0; j < TM; j++) {
-    const int gm = m0 + wm * WM + j * 32 + l32;
-    uint16_t* yrow = w.y + (int64_t)(gm < g.m ? gm : 0) * w.ldy;
-#pragma unroll
-    for (int i = 0; i < TN; i++) {
-      const int nb = n0 + wn * WN + i * 32;
-      uint32_t pk[4][2];
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
-        if (w.bias) {
-          const int nn = nb + 8 * g + 4 * hi;
-          if (nn + 3 < w.n) {
-            const uint2_t bb = *reinterpret_cast<const uint2_t*>(w.bias + nn);
-            b0 = (float)bits_to_half((uint16_t)bb[0]);
-            b1 = (float)bits_to_half((uint16_t)(bb[0] >> 16));
-            b2 = (float)bits_to_half((uint16_t)bb[1]);
-            b3 = (float)bits_to_half((uint16_t)(bb[1] >> 16));
-          } else {
-            if (nn < w.n) b0 = (float)bits_to_half(w.bias[nn]);
-            if (nn + 1 < w.n) b1 = (float)bits_to_half(w.bias[nn + 1]);
-            if (nn + 2 < w.n) b2 = (float)bits_to_half(w.bias[nn + 2]);
-          }
-        }
-        pk[g][0] = pack_h2(acc[i][j][4 * g] + b0, acc[i][j][4 * g + 1] + b1);
-        pk[g][1] = pack_h2(acc[i][j][4 * g + 2] + b2, acc[i][j][4 * g + 3] + b3);
-      }
-      // after the swaps: low half-wave holds groups 0 and 2 complete (features
-      // 0..7, 16..23), high half-wave groups 1 and 3 (features 8..15, 24..31)
-#pragma unroll
-      for (int gp = 0; gp < 2; gp++) {
-        uint32_t run[4];
-#pragma unroll
-        for (int e = 0; e < 2; e++) {
-          // v_permlane32_swap: first operand's high half <-> second operand's low half
-          auto r = __builtin_amdgcn_permlane32_swap(pk[2 * gp][e], pk[2 * gp + 1][e], false, false);
-          run[e] = r[0];      // low lanes: own group 2gp     | high lanes: low lanes' group 2gp+1
-          run[2 + e] = r[1];  // low lanes: high lanes' 2gp   | high lanes: own group 2gp+1
-        }
-        const int nn = nb + 16 * gp + 8 * hi;
-        if (gm < g.m) {
-          if (nn + 7 < w.n && ((w.ldy & 7) == 0) && ((reinterpret_cast<uintptr_t>(w.y) & 15) == 0)) {
-            *reinterpret_cast<uint4_t*>(yrow + nn) = uint4_t{run[0], run[1], run[2], run[3]};
-          } else {
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-              if (nn + e < w.n) yrow[nn + e] = (uint16_t)(run[e >> 1] >> (16 * (e & 1)));
-          }
-        }
-      }
-    }
-  }
 }
 
 
