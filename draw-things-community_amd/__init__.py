@@ -36,6 +36,7 @@ ABI_SYMBOLS = (
     "dt_dense_qx_post_f16",
     "dt_qk_norm_rope_f16",
     "dt_layernorm_modulate_f16",
+    "dt_layernorm_f16",
     "dt_sdpa_f16",
     "dt_sdpa_workspace_bytes",
 )
@@ -64,7 +65,8 @@ class _HeadEpilogue(ctypes.Structure):
 class _DensePost(ctypes.Structure):
     _fields_ = [("activation", ctypes.c_int32), ("gate", ctypes.c_void_p), ("residual", ctypes.c_void_p),
                 ("ld_residual", ctypes.c_int64), ("scale", ctypes.c_float), ("addend", ctypes.c_void_p),
-                ("ld_addend", ctypes.c_int64), ("gate_f32", ctypes.c_void_p)]
+                ("ld_addend", ctypes.c_int64), ("gate_f32", ctypes.c_void_p), ("multiplicand", ctypes.c_void_p),
+                ("ld_multiplicand", ctypes.c_int64)]
 
 
 class _DenseGroup(ctypes.Structure):
@@ -128,6 +130,8 @@ def lib():
         L.dt_qk_norm_rope_f16.argtypes = [vp, _View4, i32, i64, i32, i32, vp, f32, i32, vp, i64, f32]
         L.dt_layernorm_modulate_f16.restype = i32
         L.dt_layernorm_modulate_f16.argtypes = [vp, i64, i64, vp, i64, vp, vp, i32, f32, vp, i64]
+        L.dt_layernorm_f16.restype = i32
+        L.dt_layernorm_f16.argtypes = [vp, i64, i64, vp, i64, vp, vp, f32, vp, i64]
         L.dt_sdpa_f16.restype = i32
         L.dt_sdpa_f16.argtypes = [vp, i32, i32, i32, i32, i32, ctypes.POINTER(_Segment), i32,
                                   ctypes.POINTER(_Segment), ctypes.POINTER(_Segment), vp, vp, f32, _View4, f32,
@@ -353,20 +357,21 @@ def dense_multi(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object
     return _shape_outs(x, M, outs)
 
 
-ACT_NONE, ACT_GELU_TANH, ACT_SWISH = 0, 1, 2
+ACT_NONE, ACT_GELU_TANH, ACT_SWISH, ACT_GELU_ERF = 0, 1, 2, 3
 
 
 class DensePost:
     """Elementwise tail of one projection, in this order: scalar `scale`, fp16 `addend` [M, N] (the low-rank branch of a
-    LoRADense, Models/LoRA.swift:117-140), activation (ACT_*), per-feature fp16 gate [N], fp32 residual [M, N] that the
+    LoRADense, Models/LoRA.swift:117-140; a residual of an fp16 stream), fp16 `multiplicand` [M, N] (the gated
+    feed-forward `fc10(x) .* GELU()(fc11(x))`, Models/UNet.swift:510-513), activation (ACT_*), per-feature fp16 gate [N], fp32 residual [M, N] that the
     result is accumulated into (`x + (y .* gate).to(of: x)`, Models/Flux1.swift:250).  A float32 gate multiplies in
     fp32 on the way into the residual instead (`x + out.to(of: x) .* chunks[2]`, Models/Wan.swift:159).  With
     `residual` given and `keep_output=False` the fp16 result itself is not written."""
 
     def __init__(self, activation: int = ACT_NONE, gate=None, residual=None, keep_output: bool = True,
-                 scale: float = 1.0, addend=None):
+                 scale: float = 1.0, addend=None, multiplicand=None):
         self.activation, self.gate, self.residual, self.keep_output = activation, gate, residual, keep_output
-        self.scale, self.addend = scale, addend
+        self.scale, self.addend, self.multiplicand = scale, addend, multiplicand
 
 
 def _marshal_posts(posts, weights, M, Y, outs):
@@ -376,7 +381,7 @@ def _marshal_posts(posts, weights, M, Y, outs):
     P = (_DensePost * n)()
     for i, p in enumerate(posts):
         if p is None:
-            P[i] = _DensePost(ACT_NONE, None, None, 0, 1.0, None, 0, None)
+            P[i] = _DensePost(ACT_NONE, None, None, 0, 1.0, None, 0, None, None, 0)
             continue
         N = weights[i].shape[0]
         g16 = g32 = None
@@ -408,8 +413,15 @@ def _marshal_posts(posts, weights, M, Y, outs):
             if a2.shape != (M, N) or a2.stride(1) != 1 or a2.data_ptr() != p.addend.data_ptr():
                 raise ValueError("addend must be an [M, N] view with contiguous rows")
             ap, lda = a2.data_ptr(), a2.stride(0)
+        mp, ldm = None, 0
+        if p.multiplicand is not None:
+            m2 = _f16_cuda(p.multiplicand, "multiplicand")
+            m2 = m2.reshape(-1, N) if m2.dim() != 2 else m2
+            if m2.shape != (M, N) or m2.stride(1) != 1 or m2.data_ptr() != p.multiplicand.data_ptr():
+                raise ValueError("multiplicand must be an [M, N] view with contiguous rows")
+            mp, ldm = m2.data_ptr(), m2.stride(0)
         P[i] = _DensePost(p.activation, None if g16 is None else g16.data_ptr(), rp, ldr, float(p.scale), ap, lda,
-                          None if g32 is None else g32.data_ptr())
+                          None if g32 is None else g32.data_ptr(), mp, ldm)
     return P
 
 
@@ -609,10 +621,34 @@ def layernorm_modulate(x, scale=None, shift=None, epsilon: float = 1e-6, out=Non
     return out.reshape(tuple(x.shape[:-1]) + (C,)) if out.is_contiguous() else out
 
 
+def layernorm16(x, weight=None, bias=None, epsilon: float = 1e-5, out=None, stream=None):
+    """LayerNorm(epsilon:, axis: [last]) with fp16 affine `weight` / `bias` [C] on an fp16 tensor [..., C], fp16 out
+    (the norms of a UNet transformer block, Models/UNet.swift:530, 544, 554)."""
+    torch = _torch()
+    _f16_cuda(x, "x")
+    C = x.shape[-1]
+    x2 = x.reshape(-1, C)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    for t in (weight, bias):
+        if t is not None and (_f16_cuda(t, "weight / bias").numel() != C or not t.is_contiguous()):
+            raise ValueError("weight / bias must be contiguous vectors of C elements")
+    if out is None:
+        out = torch.empty((M, C), dtype=torch.float16, device=x.device)
+    elif out.dtype != torch.float16 or out.shape != (M, C) or out.stride(1) != 1:
+        raise ValueError("out must be an [M, C] float16 view with contiguous rows")
+    st = lib().dt_layernorm_f16(_stream_ptr(stream), M, C, x2.data_ptr(), x2.stride(0),
+                                None if weight is None else weight.data_ptr(), None if bias is None else bias.data_ptr(),
+                                float(epsilon), out.data_ptr(), out.stride(0))
+    _check("dt_layernorm_f16", st)
+    return out.reshape(tuple(x.shape[:-1]) + (C,)) if out.is_contiguous() else out
+
+
 class LayerNorm:
-    """LayerNorm(epsilon:axis:elementwiseAffine:) on the last axis of an fp32 tensor, result cast to fp16
+    """LayerNorm(epsilon:axis:elementwiseAffine:) on the last axis.  Of an fp32 tensor, result cast to fp16
     (`xNorm1(x).to(.Float16)`, Models/Flux1.swift:172-173; with fp32 `weight` / `bias` `xNorm3(out).to(.Float16)`,
-    Models/Wan.swift:160-161)."""
+    Models/Wan.swift:160-161); of an fp16 tensor with fp16 `weight` / `bias` (Models/UNet.swift:530)."""
 
     def __init__(self, epsilon: float, axis: Sequence[int], elementwiseAffine: bool = True, name: str = ""):
         self.epsilon, self.axis, self.elementwiseAffine, self.name = epsilon, list(axis), elementwiseAffine, name
@@ -622,6 +658,11 @@ class LayerNorm:
     def __call__(self, x, stream=None):
         if self.axis != [x.dim() - 1]:
             raise ValueError("LayerNorm: only the last axis is supported")
+        if x.dtype == _torch().float16:
+            if self.elementwiseAffine and (self.weight is None or self.bias is None):
+                raise RuntimeError(f"LayerNorm {self.name!r}: weight / bias not loaded")
+            return layernorm16(x, self.weight if self.elementwiseAffine else None,
+                               self.bias if self.elementwiseAffine else None, self.epsilon, stream=stream)
         if not self.elementwiseAffine:
             return layernorm_modulate(x, None, None, self.epsilon, stream=stream)
         if self.weight is None or self.bias is None:

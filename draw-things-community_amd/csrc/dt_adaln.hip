@@ -133,6 +133,101 @@ __global__ void __launch_bounds__(256) adaln_generic_kernel(const AdaLnArgs a) {
                           a.shift != nullptr, a.shift ? mod_at<MOD>(a.shift, e) : 0.f);
 }
 
+// fp16 rows with an elementwise affine weight and bias (fp16), fp16 out: lane l holds the 8 halfs at
+// element 512 i + 8 l of every 512-element chunk i.  C % 8 == 0, 16-byte aligned rows, C <= NV * 512.
+struct LayerNorm16Args {
+  const uint16_t* x;
+  int64_t ldx;
+  int64_t m, c;
+  const uint16_t* gamma;
+  const uint16_t* beta;
+  float eps;
+  uint16_t* y;
+  int64_t ldy;
+};
+
+__device__ __forceinline__ void unpack8(const uint4_t r, float (&o)[8]) {
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    o[2 * q] = (float)bits_to_half((uint16_t)r[q]);
+    o[2 * q + 1] = (float)bits_to_half((uint16_t)(r[q] >> 16));
+  }
+}
+
+template <int NV>
+__global__ void __launch_bounds__(256) layernorm16_rows_kernel(const LayerNorm16Args a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.m) return;
+  const uint16_t* xr = a.x + row * a.ldx;
+  uint16_t* yr = a.y + row * a.ldy;
+  const int c = (int)a.c;
+  float v[NV][8];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int e = i * 512 + lane * 8;
+    uint4_t r = {0u, 0u, 0u, 0u};
+    if (e < c) r = *reinterpret_cast<const uint4_t*>(xr + e);
+    unpack8(r, v[i]);
+#pragma unroll
+    for (int j = 0; j < 8; j++) s += v[i][j];
+  }
+  const float mean = wave_sum64(s) / (float)c;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    if (i * 512 + lane * 8 < c) {
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        v[i][j] -= mean;
+        q += v[i][j] * v[i][j];
+      }
+    }
+  }
+  const float inv = 1.0f / sqrtf(wave_sum64(q) / (float)c + a.eps);
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int e = i * 512 + lane * 8;
+    if (e < c) {
+      float g[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f}, b[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (a.gamma) unpack8(*reinterpret_cast<const uint4_t*>(a.gamma + e), g);
+      if (a.beta) unpack8(*reinterpret_cast<const uint4_t*>(a.beta + e), b);
+      uint32_t o[4];
+#pragma unroll
+      for (int p = 0; p < 4; p++) {
+        const uint16_t lo = half_to_bits((half_t)(v[i][2 * p] * inv * g[2 * p] + b[2 * p]));
+        const uint16_t hi = half_to_bits((half_t)(v[i][2 * p + 1] * inv * g[2 * p + 1] + b[2 * p + 1]));
+        o[p] = (uint32_t)lo | ((uint32_t)hi << 16);
+      }
+      *reinterpret_cast<uint4_t*>(yr + e) = uint4_t{o[0], o[1], o[2], o[3]};
+    }
+  }
+}
+
+// any width and alignment
+__global__ void __launch_bounds__(256) layernorm16_generic_kernel(const LayerNorm16Args a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.m) return;
+  const uint16_t* xr = a.x + row * a.ldx;
+  uint16_t* yr = a.y + row * a.ldy;
+  float s = 0.f;
+  for (int64_t e = lane; e < a.c; e += 64) s += (float)bits_to_half(xr[e]);
+  const float mean = wave_sum64(s) / (float)a.c;
+  float q = 0.f;
+  for (int64_t e = lane; e < a.c; e += 64) {
+    const float d = (float)bits_to_half(xr[e]) - mean;
+    q += d * d;
+  }
+  const float inv = 1.0f / sqrtf(wave_sum64(q) / (float)a.c + a.eps);
+  for (int64_t e = lane; e < a.c; e += 64) {
+    const float n = ((float)bits_to_half(xr[e]) - mean) * inv;
+    const float g = a.gamma ? (float)bits_to_half(a.gamma[e]) : 1.f, b = a.beta ? (float)bits_to_half(a.beta[e]) : 0.f;
+    yr[e] = half_to_bits((half_t)(n * g + b));
+  }
+}
+
 template <int MOD>
 static void launch_adaln(hipStream_t s, const AdaLnArgs& a, bool vec) {
   const dim3 grid((unsigned)((a.m + 3) / 4)), block(256);
@@ -174,3 +269,30 @@ DT_EXPORT dt_status dt_layernorm_modulate_f16(dt_stream stream, int64_t M, int64
   else launch_adaln<DT_MOD_AFFINE_F32>(as_stream(stream), a, vec);
   return launch_status();
 }
+
+DT_EXPORT dt_status dt_layernorm_f16(dt_stream stream, int64_t M, int64_t C, const uint16_t* X, int64_t ldx,
+                                     const uint16_t* gamma, const uint16_t* beta, float eps, uint16_t* Y, int64_t ldy) {
+  using namespace dt;
+  if (M < 0 || C <= 0) return DT_INVALID;
+  if (!(eps >= 0.f) || eps - eps != 0.f) return DT_INVALID;
+  if (M == 0) return DT_OK;
+  if (!X || !Y || ldx < C || ldy < C) return DT_INVALID;
+  if (((reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Y) | reinterpret_cast<uintptr_t>(gamma) |
+        reinterpret_cast<uintptr_t>(beta)) & 1) != 0)
+    return DT_INVALID;
+  if ((M + 3) / 4 > 0x7fffffff) return DT_NO_KERNEL;
+  if (!device_ok()) return DT_NO_KERNEL;
+  const LayerNorm16Args a{X, ldx, M, C, gamma, beta, eps, Y, ldy};
+  const bool vec = (C % 8 == 0) && (ldx % 8 == 0) && (ldy % 8 == 0) && C <= 8 * 512 &&
+                   ((reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Y) | reinterpret_cast<uintptr_t>(gamma) |
+                     reinterpret_cast<uintptr_t>(beta)) & 15) == 0;
+  const dim3 grid((unsigned)((M + 3) / 4)), block(256);
+  hipStream_t s = as_stream(stream);
+  if (!vec) hipLaunchKernelGGL(layernorm16_generic_kernel, grid, block, 0, s, a);
+  else if (C <= 512) hipLaunchKernelGGL((layernorm16_rows_kernel<1>), grid, block, 0, s, a);
+  else if (C <= 1024) hipLaunchKernelGGL((layernorm16_rows_kernel<2>), grid, block, 0, s, a);
+  else if (C <= 2048) hipLaunchKernelGGL((layernorm16_rows_kernel<4>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((layernorm16_rows_kernel<8>), grid, block, 0, s, a);
+  return launch_status();
+}
+

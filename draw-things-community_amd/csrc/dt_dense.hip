@@ -23,7 +23,8 @@ __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* _
                                                              uint16_t* y, int64_t ldy, float scale,
                                                              const uint16_t* add, int64_t ld_add, int act,
                                                              const uint16_t* __restrict__ gate, float* __restrict__ res,
-                                                             int64_t ld_res, const float* __restrict__ gate32) {
+                                                             int64_t ld_res, const float* __restrict__ gate32,
+                                                             const uint16_t* mul, int64_t ld_mul) {
   int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (o >= m * n) return;
   int64_t mi = o / n, ni = o - mi * n;
@@ -45,7 +46,8 @@ __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* _
   }
   if (bias) acc += (float)bits_to_half(bias[ni]);
   float v = (float)(half_t)acc;
-  v = post_value(v, scale, add != nullptr, add ? (float)bits_to_half(add[mi * ld_add + ni]) : 0.f, act, gate != nullptr,
+  v = post_value(v, scale, add != nullptr, add ? (float)bits_to_half(add[mi * ld_add + ni]) : 0.f, mul != nullptr,
+                 mul ? (float)bits_to_half(mul[mi * ld_mul + ni]) : 1.f, act, gate != nullptr,
                  gate ? (float)bits_to_half(gate[ni]) : 1.0f);
   if (res) {
     float pr = gate32 ? v * gate32[ni] : v;
@@ -65,7 +67,7 @@ extern template dt_status launch_dense_q<16>(hipStream_t, const DenseArgs&, int,
 // the kernel with the elementwise tail only when some weight of the launch asks for one
 static dt_status launch_dense(hipStream_t s, const DenseArgs& a, int tile, int qbits, int mode) {
   bool post = false;
-  for (int i = 0; i < kMaxWeights; i++) post = post || a.w[i].act != DT_ACT_NONE || a.w[i].gate || a.w[i].res || a.w[i].add || a.w[i].scale != 1.0f;
+  for (int i = 0; i < kMaxWeights; i++) post = post || a.w[i].act != DT_ACT_NONE || a.w[i].gate || a.w[i].res || a.w[i].add || a.w[i].mul || a.w[i].scale != 1.0f;
   switch (qbits) {
     case 4: return launch_dense_q<4>(s, a, tile, post, mode);
     case 5: return launch_dense_q<5>(s, a, tile, post, mode);
@@ -139,7 +141,9 @@ static dt_status validate_group(const HostGroup& h) {
   if (h.post)
     for (int i = 0; i < h.n_weights; i++) {
       const dt_dense_post& p = h.post[i];
-      if (p.activation < DT_ACT_NONE || p.activation > DT_ACT_SWISH) return DT_INVALID;
+      if (p.activation < DT_ACT_NONE || p.activation > DT_ACT_GELU_ERF) return DT_INVALID;
+      if (p.multiplicand && ((reinterpret_cast<uintptr_t>(p.multiplicand) & 1) || (h.W && h.K > 0 && p.ld_multiplicand < h.W[i].count / h.K)))
+        return DT_INVALID;
       if (p.residual && ((reinterpret_cast<uintptr_t>(p.residual) & 3) || (h.W && h.K > 0 && p.ld_residual < h.W[i].count / h.K)))
         return DT_INVALID;
       if (p.addend && ((reinterpret_cast<uintptr_t>(p.addend) & 1) || (h.W && h.K > 0 && p.ld_addend < h.W[i].count / h.K)))
@@ -207,6 +211,8 @@ static int add_weight(DenseArgs& a, int slot, const HostGroup& h, int wi, int ti
   d.res = h.post ? h.post[wi].residual : nullptr;
   d.ld_res = h.post ? h.post[wi].ld_residual : 0;
   d.gate32 = h.post ? h.post[wi].gate_f32 : nullptr;
+  d.mul = h.post ? h.post[wi].multiplicand : nullptr;
+  d.ld_mul = h.post ? h.post[wi].ld_multiplicand : 0;
   return (int)((n_rows + BN - 1) / BN);
 }
 
@@ -239,7 +245,8 @@ static dt_status run_group(hipStream_t s, const HostGroup& h) {
                            h.post ? h.post[i].addend : nullptr, h.post ? h.post[i].ld_addend : 0,
                            h.post ? h.post[i].activation : DT_ACT_NONE,
                            h.post ? h.post[i].gate : nullptr, h.post ? h.post[i].residual : nullptr,
-                           h.post ? h.post[i].ld_residual : 0, h.post ? h.post[i].gate_f32 : nullptr);
+                           h.post ? h.post[i].ld_residual : 0, h.post ? h.post[i].gate_f32 : nullptr,
+                           h.post ? h.post[i].multiplicand : nullptr, h.post ? h.post[i].ld_multiplicand : 0);
         dt_status st = launch_status();
         if (st != DT_OK) return st;
         if (h.wants_epi(i)) {

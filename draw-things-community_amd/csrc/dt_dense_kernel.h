@@ -44,6 +44,8 @@ struct DenseWeight {
   float* res;            // [m, n] fp32 with row stride ld_res, updated in place; null = none
   int64_t ld_res;
   const float* gate32;   // [n] fp32 or null: the residual receives float(result) * gate32 (no fp16 product)
+  const uint16_t* mul;   // [m, n] fp16 with row stride ld_mul, multiplies the result; null = none
+  int64_t ld_mul;
 };
 
 // The elementwise tail on one value that has already been rounded to fp16, with
@@ -58,12 +60,15 @@ __device__ __forceinline__ float act_gelu_tanh(float x) {
 __device__ __forceinline__ float act_swish(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
 }
-__device__ __forceinline__ float post_value(float v, float scale, bool has_add, float add, int act, bool has_gate,
-                                            float gate) {
+__device__ __forceinline__ float act_gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f)); }
+__device__ __forceinline__ float post_value(float v, float scale, bool has_add, float add, bool has_mul, float mul, int act,
+                                            bool has_gate, float gate) {
   if (scale != 1.0f) v = (float)(half_t)(v * scale);
   if (has_add) v = (float)(half_t)(v + add);
+  if (has_mul) v = (float)(half_t)(v * mul);
   if (act == DT_ACT_GELU_TANH) v = (float)(half_t)act_gelu_tanh(v);
   else if (act == DT_ACT_SWISH) v = (float)(half_t)act_swish(v);
+  else if (act == DT_ACT_GELU_ERF) v = (float)(half_t)act_gelu_erf(v);
   if (has_gate) v = (float)(half_t)(v * gate);
   return v;
 }
@@ -680,6 +685,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // what a row needs from memory before its arithmetic
   struct RowIn {
     uint4_t add;  // the addend, or the RoPE table row of a head tile
+    uint4_t mul;
     float4_t r0, r1;
   };
   // FAST: the wave's slice lies inside the matrix and every row meets the vector alignment
@@ -691,6 +697,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
       if (head && w.rot) in.add = *reinterpret_cast<const uint4_t*>(w.rot + (w.rot_pos0 + gm) * WN + 8 * c);
       if constexpr (POST) {
         if (w.add) in.add = *reinterpret_cast<const uint4_t*>(w.add + gm * w.ld_add + nn);
+        if (w.mul) in.mul = *reinterpret_cast<const uint4_t*>(w.mul + gm * w.ld_mul + nn);
         if (w.res) {
           in.r0 = *reinterpret_cast<const float4_t*>(w.res + gm * w.ld_res + nn);
           in.r1 = *reinterpret_cast<const float4_t*>(w.res + gm * w.ld_res + nn + 4);
@@ -756,6 +763,20 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
               if (nn + e < w.n) ad[e] = (float)bits_to_half(w.add[gmc * w.ld_add + nn + e]);
           }
         }
+        float ml[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
+        if (w.mul) {
+          if constexpr (FAST) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              ml[2 * q] = lo16(cur.mul[q]);
+              ml[2 * q + 1] = hi16(cur.mul[q]);
+            }
+          } else if (row_ok) {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              if (nn + e < w.n) ml[e] = (float)bits_to_half(w.mul[gmc * w.ld_mul + nn + e]);
+          }
+        }
         if (w.res) {
           if constexpr (FAST) {
 #pragma unroll
@@ -771,7 +792,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         }
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-          v[e] = post_value(v[e], w.scale, w.add != nullptr, ad[e], w.act, w.gate != nullptr, gt[e]);
+          v[e] = post_value(v[e], w.scale, w.add != nullptr, ad[e], w.mul != nullptr, ml[e], w.act, w.gate != nullptr, gt[e]);
           float pr = w.gate32 ? v[e] * gt[e] : v[e];  // the fp32 gate's product is its own op: rounded before the addition
           asm volatile("" : "+v"(pr));
           res[e] += pr;
@@ -802,6 +823,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const bool aligned16 = (!w.y || (((w.ldy & 7) == 0) && (reinterpret_cast<uintptr_t>(w.y) & 15) == 0)) &&
                          (!(head && w.rot) || (reinterpret_cast<uintptr_t>(w.rot) & 15) == 0) &&
                          (!POST || ((!w.add || (((w.ld_add & 7) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 15) == 0)) &&
+                                    (!w.mul || (((w.ld_mul & 7) == 0) && (reinterpret_cast<uintptr_t>(w.mul) & 15) == 0)) &&
                                     (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0))));
   if (aligned16 && nw + WN <= w.n && m0 + wm * WM + WM <= g.m) walk(std::true_type{});
   else walk(std::false_type{});

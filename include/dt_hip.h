@@ -156,8 +156,11 @@ dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K, const ui
  *   scale      : scalar multiplier of the result; 0 or 1 = none (configuration.scale * downX, Models/LoRA.swift:129-134)
  *   addend     : fp16 [M, N_i] with row stride ld_addend, added to the result: the low-rank branch of a
  *                LoRADense, out = dense(x) + up(down(x)) (Models/LoRA.swift:117-140); may be Y[i] itself (in place)
+ *   multiplicand : fp16 [M, N_i] with row stride ld_multiplicand, multiplies the result elementwise: the gated
+ *                feed-forward fc10(x) .* GELU()(fc11(x)) (Models/UNet.swift:510-513); may be Y[i] itself
  *   activation : DT_ACT_GELU_TANH  linear1(x).GELU(approximate: .tanh)  (Models/Flux1.swift:133-135, Models/Wan.swift:52-53)
  *                DT_ACT_SWISH      fc0(x).swish()                       (Models/Flux1.swift:122-123)
+ *                DT_ACT_GELU_ERF   GELU()(fc11(x)), the erf form          (Models/UNet.swift:513)
  *   gate       : [N_i] fp16, multiplies every output row ((xOut .* xChunks[2]), Models/Flux1.swift:246-250)
  *   residual   : fp32 [M, N_i] with row stride ld_residual, updated in place:
  *                residual += float(result)  (x + (...).to(of: x), Models/Flux1.swift:250, 275-283)
@@ -171,6 +174,7 @@ dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K, const ui
 #define DT_ACT_NONE 0
 #define DT_ACT_GELU_TANH 1
 #define DT_ACT_SWISH 2
+#define DT_ACT_GELU_ERF 3
 
 typedef struct {
   int32_t activation;
@@ -181,6 +185,8 @@ typedef struct {
   const uint16_t* addend;
   int64_t ld_addend;
   const float* gate_f32;
+  const uint16_t* multiplicand;
+  int64_t ld_multiplicand;
 } dt_dense_post;
 
 dt_status dt_dense_qx_post_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,
@@ -204,6 +210,15 @@ dt_status dt_dense_qx_post_f16(dt_stream stream, int64_t M, int64_t K, const uin
  * aligned with C % 4 == 0 and C <= 8192 stay in registers (one read, one write);
  * anything else takes a three-pass kernel with the same results.
  */
+/*
+ * LayerNorm(epsilon:, axis: [last]) with its elementwise affine weight and bias on an fp16 tensor, fp16 out:
+ * the norms of a UNet transformer block (LayerNorm(epsilon: 1e-5, axis: [2]), Models/UNet.swift:530, 544, 554).
+ * Statistics and the affine step in fp32, one rounding at the end.  gamma / beta: fp16 [C], may be NULL.
+ * Y may be X (in place).
+ */
+dt_status dt_layernorm_f16(dt_stream stream, int64_t M, int64_t C, const uint16_t* X, int64_t ldx,
+                           const uint16_t* gamma, const uint16_t* beta, float eps, uint16_t* Y, int64_t ldy);
+
 #define DT_MOD_F16 0
 #define DT_MOD_F32 1
 #define DT_MOD_AFFINE_F32 2

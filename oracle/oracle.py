@@ -353,6 +353,33 @@ def np_gelu_tanh16(y16: np.ndarray) -> np.ndarray:
     return (np.float32(0.5) * x * (np.float32(1) + np.tanh(u))).astype(np.float16)
 
 
+def np_gelu_erf16(y16: np.ndarray) -> np.ndarray:
+    """GELU() in its erf form, 0.5 x (1 + erf(x / sqrt 2)) (GELU()(fc11(x)), Models/UNet.swift:513), fp16 in and out."""
+    from scipy.special import erf
+    x = y16.astype(np.float64)
+    return (0.5 * x * (1 + erf(x / np.sqrt(2.0)))).astype(np.float32).astype(np.float16)
+
+
+def np_mul16(a16: np.ndarray, b16: np.ndarray) -> np.ndarray:
+    """fp16 elementwise product (out .* GELU()(fc11(x)), Models/UNet.swift:513): the float32 product of two fp16 values
+    is exact, so one rounding."""
+    return (a16.astype(np.float32) * b16.astype(np.float32)).astype(np.float16)
+
+
+def np_layernorm16(x16: np.ndarray, gamma16=None, beta16=None, eps: float = 1e-5) -> np.ndarray:
+    """LayerNorm(epsilon:, axis: [last]) with fp16 affine weight and bias on an fp16 tensor (Models/UNet.swift:530,
+    544, 554): statistics (biased variance) and the affine step in float64, one rounding to fp16 at the end."""
+    x = x16.astype(np.float64)
+    mean = x.mean(axis=-1, keepdims=True)
+    var = ((x - mean) ** 2).mean(axis=-1, keepdims=True)
+    y = (x - mean) / np.sqrt(var + eps)
+    if gamma16 is not None:
+        y = y * gamma16.astype(np.float64)
+    if beta16 is not None:
+        y = y + beta16.astype(np.float64)
+    return y.astype(np.float32).astype(np.float16)
+
+
 def np_swish16(y16: np.ndarray) -> np.ndarray:
     x = y16.astype(np.float32)
     return (x / (np.float32(1) + np.exp(-x))).astype(np.float16)
@@ -484,4 +511,28 @@ def np_flux_single_block(x32, rot16, xch, dense, norm, k, h):
     att = C.sdpa(Q_[None], K_[None], V_[None], 1.0 / np.sqrt(k))[0].reshape(S, h * k)
     ff = dense["x_out_proj"](np_gelu_tanh16(dense["x_linear1"](xn)))
     return np_gated_residual(x32, np_add16(dense["x_o"](att), ff), xch[2])
+
+
+def np_unet_transformer_block(x16, c16, dense, norm, k, h):
+    """BasicTransformerBlock of the SD 1.5 UNet op by op (Models/UNet.swift:519-565; fp16, no injected KV / IP
+    adapters): LayerNorm(1e-5) with affine (:530, 538), self-attention q / k / v without bias and attention at
+    1 / sqrt(k) with the unify-heads projection (:95-156), + x (:542), LayerNorm, cross-attention with keys and values
+    from the text context (:269-320), + residual (:551), LayerNorm, fc10(x) .* GELU()(fc11(x)) -> fc2 (:506-517),
+    + residual (:558).  x16 [b, hw, C], c16 [b, t, Cc]; `dense[name]`: callable X16 -> Y16; `norm[name]`: (weight,
+    bias) fp16."""
+    b, hw, C_ = x16.shape
+    t = c16.shape[1]
+    x2 = x16.reshape(b * hw, C_)
+    c2 = c16.reshape(b * t, c16.shape[2])
+    scale = 1.0 / np.sqrt(k)
+    heads = lambda y, s: y.reshape(b, s, h, k)
+    n1 = np_layernorm16(x2, *norm["layerNorm1"], 1e-5)
+    att = C.sdpa(heads(dense["toqueries1"](n1), hw), heads(dense["tokeys1"](n1), hw), heads(dense["tovalues1"](n1), hw), scale)
+    out = np_add16(dense["unifyheads1"](att.reshape(b * hw, C_)), x2)
+    n2 = np_layernorm16(out, *norm["layerNorm2"], 1e-5)
+    att = C.sdpa(heads(dense["toqueries2"](n2), hw), heads(dense["tokeys2"](c2), t), heads(dense["tovalues2"](c2), t), scale)
+    out = np_add16(dense["unifyheads2"](att.reshape(b * hw, C_)), out)
+    n3 = np_layernorm16(out, *norm["layerNorm3"], 1e-5)
+    hid = np_mul16(dense["fc10"](n3), np_gelu_erf16(dense["fc11"](n3)))
+    return np_add16(dense["fc2"](hid), out).reshape(b, hw, C_)
 

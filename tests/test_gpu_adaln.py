@@ -103,3 +103,31 @@ def test_layernorm_modulate_flux_full_size(dthip, oracle):
         got = dthip.layernorm_modulate(x, torch.from_numpy(scale).cuda(), torch.from_numpy(shift).cuda(), 1e-6)
         want = oracle.np_layernorm_modulate16(x[rows].cpu().numpy(), scale, shift, 1e-6, mod)
         assert close(got[rows].cpu().numpy(), want, shift)
+
+
+@pytest.mark.parametrize("M,C", [(9, 320), (300, 1280), (5, 4096), (7, 100), (3, 4104), (2, 8)])
+def test_layernorm16_vs_oracle(dthip, oracle, M, C):
+    """LayerNorm with fp16 affine weight and bias on an fp16 tensor (the UNet block's norms): one fp16 ulp of the
+    oracle's float64 statement (two where the affine step cancels); strided views; in place."""
+    import torch
+    rng = np.random.default_rng(M + C)
+    x = (rng.standard_normal((M, C)) * 2 + 0.5).astype(np.float16)
+    g = (1 + 0.2 * rng.standard_normal(C)).astype(np.float16)
+    b = (0.3 * rng.standard_normal(C)).astype(np.float16)
+    xd, gd, bd = (torch.from_numpy(a).cuda() for a in (x, g, b))
+    print("layernorm16", M, C, flush=True)
+    assert close(dthip.layernorm16(xd, gd, bd, 1e-5).cpu().numpy(), oracle.np_layernorm16(x, g, b, 1e-5), b)
+    assert close(dthip.layernorm16(xd, None, None, 1e-5).cpu().numpy(), oracle.np_layernorm16(x, None, None, 1e-5))
+    big = torch.zeros((M, C + 16), dtype=torch.float16, device="cuda")
+    big[:, 8:8 + C].copy_(xd)
+    out = torch.full((M, C + 16), 3.0, dtype=torch.float16, device="cuda")
+    dthip.layernorm16(big[:, 8:8 + C], gd, bd, 1e-5, out=out[:, 8:8 + C])
+    assert torch.equal(out[:, 8:8 + C], dthip.layernorm16(xd, gd, bd, 1e-5))
+    assert float((out[:, :8] - 3).abs().max()) == 0 and float((out[:, 8 + C:] - 3).abs().max()) == 0
+    same = xd.clone()
+    dthip.layernorm16(same, gd, bd, 1e-5, out=same)
+    assert torch.equal(same, dthip.layernorm16(xd, gd, bd, 1e-5))
+    ln = dthip.LayerNorm(1e-5, [1])
+    ln.weight, ln.bias = gd, bd
+    assert torch.equal(ln(xd), dthip.layernorm16(xd, gd, bd, 1e-5))
+

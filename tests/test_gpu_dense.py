@@ -489,6 +489,35 @@ def test_dense_grouped_with_tails_equals_separate(dthip, oracle, torch_cuda):
         dthip.dense_grouped([dict(x=x, weights=[wh], biases=[None], epilogues=[epi], posts=[dthip.DensePost()])])
 
 
+@pytest.mark.parametrize("M,N,K,q,nib", [(1100, 384, 128, 6, 4096), (70, 100, 96, 6, 64), (300, 320, 320, 16, 0)])
+def test_dense_post_multiplicand_and_erf_gelu(dthip, oracle, torch_cuda, M, N, K, q, nib):
+    """The gated feed-forward of the UNet block, fc10(x) .* GELU()(fc11(x)): the product step bit for bit on the
+    device's own Dense result (in place over the multiplicand too), the erf GELU within one fp16 ulp."""
+    torch = torch_cuda
+    rng = np.random.default_rng(M + K)
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    if q == 16:
+        w = dthip.QxTensor.from_f16((rng.standard_normal((N, K)) * 0.05).astype(np.float16))
+    else:
+        w, _ = make_weight(dthip, oracle, rng, N, K, q, nib, std=0.05)
+    bias = to_dev(torch, (rng.standard_normal(N) * 0.1).astype(np.float16))
+    xd = to_dev(torch, X)
+    print("dense multiplicand", M, N, K, q, flush=True)
+    plain = dthip.dense_multi(xd, [w], [bias])[0]
+    g = dthip.dense_post(xd, [w], [bias], [dthip.DensePost(dthip.ACT_GELU_ERF)])[0]
+    got, want = g.cpu().numpy(), oracle.np_gelu_erf16(plain.cpu().numpy())
+    tol = np.maximum(np.spacing(np.abs(want)).astype(np.float32), np.float32(2.0 ** -19))
+    assert np.all(np.abs(got.astype(np.float32) - want.astype(np.float32)) <= tol)
+    m = to_dev(torch, rng.standard_normal((M, N)).astype(np.float16))
+    prod = dthip.dense_post(xd, [w], [bias], [dthip.DensePost(multiplicand=m)])[0]
+    assert np.array_equal(prod.cpu().numpy().view(np.uint16), oracle.np_mul16(plain.cpu().numpy(), m.cpu().numpy()).view(np.uint16))
+    buf = m.clone()
+    dthip.dense_post(xd, [w], [bias], [dthip.DensePost(multiplicand=buf)], outs=[buf])
+    assert torch.equal(buf, prod)
+    with pytest.raises(ValueError):
+        dthip.dense_post(xd, [w], [bias], [dthip.DensePost(multiplicand=m[:, :-1])])
+
+
 def test_dense_post_bad_args(dthip, oracle, torch_cuda):
     torch = torch_cuda
     rng = np.random.default_rng(9)

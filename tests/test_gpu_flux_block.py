@@ -175,3 +175,45 @@ def test_joint_block_replays_as_hip_graph(dthip, oracle):
         torch.cuda.synchronize()
         assert torch.equal(again_c, want_c) and torch.equal(again_x, want_x)
 
+
+@pytest.mark.parametrize("k,h,b,gs,t,cw,q", [(40, 8, 2, 32, 77, 768, 6), (64, 2, 1, 7, 10, 96, 16)])
+def test_unet_transformer_block_vs_oracle(dthip, oracle, k, h, b, gs, t, cw, q):
+    """A whole SD 1.5 transformer block (fp16 stream: affine LayerNorms, self- and cross-attention with head dimension
+    40, the erf-GELU gated feed-forward, fp16 residual additions in the Dense epilogues) against the oracle's
+    op-by-op restatement of Models/UNet.swift:519-565.  q = 16: plain fp16 weights."""
+    import torch
+    unet = importlib.import_module(dthip.__name__ + ".unet")
+    hw, C = gs * gs, h * k
+    inter = 4 * C
+    rng = np.random.default_rng(C + hw)
+    blk = unet.BasicTransformerBlock(k, h, b, hw, t)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    dense, norm = {}, {}
+    for name in unet.DENSE_NAMES:
+        K = cw if name in ("tokeys2", "tovalues2") else inter if name == "fc2" else C
+        N = inter if name in ("fc10", "fc11") else C
+        bias = None if name in unet.NO_BIAS else (rng.standard_normal(N) * 0.05).astype(np.float16)
+        if q == 16:
+            Wh = (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float16)
+            blk.weight[name] = dthip.QxTensor.from_f16(Wh)
+            dense[name] = (lambda w_, bb: (lambda X: oracle.C.dense(np.ascontiguousarray(X), w_, bb)))(Wh, bias)
+        else:
+            packed, _, _ = oracle.synth_qx_weight(rng, N, K, q, 4096, 1.0 / np.sqrt(K))
+            blk.weight[name] = dthip.QxTensor.from_packed(packed, q, 4096, (N, K))
+            dense[name] = (lambda p, n, bb: (lambda X: oracle.C.dense_qx(np.ascontiguousarray(X), p, q, 4096, n, bb)))(packed, N, bias)
+        if bias is not None:
+            blk.bias[name] = dev(bias)
+    for name in unet.NORM_NAMES:
+        g = (1 + 0.1 * rng.standard_normal(C)).astype(np.float16)
+        bb = (0.1 * rng.standard_normal(C)).astype(np.float16)
+        blk.norm[name] = (dev(g), dev(bb))
+        norm[name] = (g, bb)
+    x = rng.standard_normal((b, hw, C)).astype(np.float16)
+    c = rng.standard_normal((b, t, cw)).astype(np.float16)
+    print("unet block", k, h, b, hw, t, q, flush=True)
+    got = blk(dev(x), dev(c)).cpu().numpy()
+    want = oracle.np_unet_transformer_block(x, c, dense, norm, k, h)
+    mx, rr = oracle.err_stats(got, want)
+    print("x max-abs", mx, "rel-rms", rr, "scale", float(np.abs(want.astype(np.float32)).max()), flush=True)
+    assert mx <= 2e-2 and rr <= 2e-3
+

@@ -368,3 +368,33 @@ def test_layernorm_modulate_pinned(oracle):
                           np.array([[np.float32(1) + np.float32(1.0009765625) ** 2, 0.5]], np.float32))
     assert np.array_equal(oracle.np_gated_residual32(res, y), res + y.astype(np.float32))
 
+
+def test_unet_block_pieces_pinned(oracle):
+    """The fp16 LayerNorm with affine, the erf GELU and the fp16 product against library routines and closed forms."""
+    import math
+    import torch
+    rng = np.random.default_rng(21)
+    x = (rng.standard_normal((5, 320)) * 2 + 0.3).astype(np.float16)
+    g = (1 + 0.2 * rng.standard_normal(320)).astype(np.float16)
+    b = (0.3 * rng.standard_normal(320)).astype(np.float16)
+    got = oracle.np_layernorm16(x, g, b, 1e-5).astype(np.float64)
+    ref = torch.nn.functional.layer_norm(torch.from_numpy(x.astype(np.float32)), (320,), torch.from_numpy(g.astype(np.float32)),
+                                         torch.from_numpy(b.astype(np.float32)), 1e-5).numpy().astype(np.float64)
+    assert np.max(np.abs(got - ref)) <= 2.0 ** -10 * np.maximum(1, np.abs(ref)).max()
+    # weight 1 / bias 0 equals no affine; a constant row gives the bias alone
+    assert np.array_equal(oracle.np_layernorm16(x, None, None, 1e-5),
+                          oracle.np_layernorm16(x, np.ones(320, np.float16), np.zeros(320, np.float16), 1e-5))
+    assert np.array_equal(oracle.np_layernorm16(np.full((1, 320), 2.5, np.float16), g, b, 1e-5), b[None, :])
+    # erf GELU: torch's exact form; gelu(x) - gelu(-x) = x; it differs from the tanh form (by up to ~5e-4 around |x| = 2)
+    t = np.linspace(-6, 6, 2401).astype(np.float16)
+    ge = oracle.np_gelu_erf16(t).astype(np.float64)
+    ref = torch.nn.functional.gelu(torch.from_numpy(t.astype(np.float64))).numpy()
+    assert np.max(np.abs(ge - ref)) <= 2.0 ** -11 * np.maximum(1, np.abs(ref)).max()
+    assert np.max(np.abs((ge - ge[::-1]) - t.astype(np.float64))) <= 4e-3
+    assert abs(float(oracle.np_gelu_erf16(np.array([1.0], np.float16))[0]) - 0.5 * (1 + math.erf(1 / math.sqrt(2)))) < 1e-3
+    assert np.max(np.abs(ge - oracle.np_gelu_tanh16(t).astype(np.float64))) > 1e-4
+    # fp16 product: exact where representable, one rounding otherwise
+    a = np.array([1.5, 3.0, 1.0009765625], np.float16)
+    c = np.array([2.0, 0.5, 1.0009765625], np.float16)
+    assert np.array_equal(oracle.np_mul16(a, c), np.array([3.0, 1.5, 1.001953125], np.float16))
+
