@@ -228,6 +228,9 @@ static void finish_args(DenseArgs& a, int n_groups, int n_w, int64_t K, const dt
 // One validated problem with M > 0: weights that share (qbits, nib) and meet the
 // tiled kernel's alignment go out in runs of up to kMaxWeights per launch; the
 // rest take the generic kernel.
+// Fewer 256 x 256 tiles than this leave too many of the 256 compute units idle: such launches take 128 x 128 tiles.
+constexpr int64_t kFillTiles = 192;
+
 static dt_status run_group(hipStream_t s, const HostGroup& h) {
   const int64_t M = h.M, K = h.K;
   const bool x_ok = h.x_ok();
@@ -261,7 +264,14 @@ static dt_status run_group(hipStream_t s, const HostGroup& h) {
     bool any_fused = false;
     for (int j = i; j < h.n_weights && j < i + kMaxWeights; j++)
       any_fused = any_fused || (h.wants_epi(j) && h.fusable(j));
-    const bool big = ((M >= 1024) && (n_rows0 >= 256)) || any_fused;  // the fused epilogue needs the 128-feature wave slice
+    // (the fused epilogue needs the 128-feature wave slice of the big tile)
+    int64_t big_tiles = 0;  // 256 x 256 tiles this launch would have
+    for (int j = i, cnt = 0; j < h.n_weights && cnt < kMaxWeights; j++, cnt++) {
+      const dt_qx_weight& wj = h.W[j];
+      if (wj.qbits != w0.qbits || (wj.qbits != 16 && wj.nib != w0.nib) || !h.w_tiled(j)) break;
+      big_tiles += ((M + 255) / 256) * ((wj.count / K + 255) / 256);
+    }
+    const bool big = ((M >= 1024) && (n_rows0 >= 256) && big_tiles >= kFillTiles) || any_fused;
     // few token rows: halve the token tile so that more workgroups share the work
     const bool narrow = big && M < 1024;
     const int BM = big ? (narrow ? 128 : 256) : 128, BN = big ? 256 : 128;
