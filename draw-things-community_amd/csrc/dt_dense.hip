@@ -115,12 +115,16 @@ struct HostGroup {
            (!epi[wi].rot || (reinterpret_cast<uintptr_t>(epi[wi].rot) & 7) == 0) &&
            (!bias || !bias[wi] || (reinterpret_cast<uintptr_t>(bias[wi]) & 7) == 0);
   }
+  // (the tiled kernel addresses X and the packed weight with 32-bit byte offsets from their bases)
   bool x_ok() const {
-    return (K % (2 * BK) == 0) && (ldx % 8 == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
+    return (K % (2 * BK) == 0) && (ldx % 8 == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0) &&
+           (M == 0 || ((M - 1) * ldx + K) * 2 <= (int64_t)0xffffffff);
   }
   bool w_tiled(int wi) const {
     const dt_qx_weight& w = W[wi];
-    return w.count / K > 0 && (reinterpret_cast<uintptr_t>(w.data) & 15) == 0 && (w.qbits == 16 || w.nib % 32 == 0);
+    if (!(w.count / K > 0 && (reinterpret_cast<uintptr_t>(w.data) & 15) == 0 && (w.qbits == 16 || w.nib % 32 == 0))) return false;
+    const int64_t bytes = w.qbits == 16 ? w.count * 2 : dt_qx_bytes(w.qbits, w.nib, w.count);
+    return bytes > 0 && bytes <= (int64_t)0xffffffff;
   }
 };
 

@@ -165,6 +165,24 @@ def test_dense_special_cases(dthip, oracle, torch_cuda):
     assert dthip.Dense.__call__(d, torch.zeros((0, K), dtype=torch.float16, device="cuda")).shape == (0, N)
 
 
+def test_dense_rows_beyond_4gib(dthip, oracle, torch_cuda):
+    """X rows spread over more than 4 GiB (a view with a huge row stride): the tiled kernel's 32-bit byte offsets do
+    not reach, so the call takes the any-shape kernel -- same results as the compact copy of the same rows."""
+    torch = torch_cuda
+    rng = np.random.default_rng(12)
+    K, N, ld = 128, 192, (1 << 30) + 8
+    w, packed = make_weight(dthip, oracle, rng, N, K, 6, 4096, std=0.05)
+    rows = rng.standard_normal((3, K)).astype(np.float16)
+    big = torch.empty(2 * ld + K, dtype=torch.float16, device="cuda")
+    view = torch.as_strided(big, (3, K), (ld, 1))
+    view.copy_(to_dev(torch, rows))
+    print("dense rows beyond 4 GiB", flush=True)
+    got = dthip.dense_multi(view, [w], [None])[0].cpu().numpy()
+    mx, rr = oracle.err_stats(got, oracle.C.dense_qx(rows, packed, 6, 4096, N, None))
+    assert mx <= MAX_ABS and rr <= REL_RMS
+    del big, view
+
+
 def test_dense_rejects_bad_arguments(dthip, torch_cuda):
     torch = torch_cuda
     w = dthip.QxTensor(torch.zeros(1024, dtype=torch.uint8, device="cuda"), 3, 32, (4, 32))
