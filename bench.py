@@ -28,8 +28,10 @@ MEASURED_TRAFFIC_BYTES = {"dense_qkv": 4.715e8, "sdpa": 1.326e8}
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # One step is ~0.7 ms; the card needs ~50 ms of continuous work to reach its sustained clock, so the default
+    # warm-up is 100 steps.  Fewer than that measures the clock ramp (about 6 % slower), not the kernels.
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch the step's kernels one by one instead of as a HIP graph")
     ap.add_argument("--kernel-iters", type=int, default=20, help="launches per kernel for the per-kernel timings")
