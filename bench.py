@@ -34,7 +34,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch the step's kernels one by one instead of as a HIP graph")
-    ap.add_argument("--kernel-iters", type=int, default=20, help="launches per kernel for the per-kernel timings")
+    ap.add_argument("--kernel-iters", type=int, default=50, help="launches per kernel for the per-kernel timings")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -128,6 +128,14 @@ def main():
         k_sdpa()
         k_out()
 
+    # inputs of the per-kernel legs, made here so that no host work (and no idle GPU) sits between the timed loops
+    x_all = f16((S, C))
+    y3 = [torch.empty((S, C), dtype=torch.float16, device=dev) for _ in range(3)]
+    wf16 = pkg.QxTensor.from_f16(w["x_q"].dequantize())
+    x32 = torch.randn((S, C), dtype=torch.float32, device=dev)
+    ln_out = torch.empty((S, C), dtype=torch.float16, device=dev)
+    ln_scale, ln_shift = f16((C,), 0.2), f16((C,), 0.2)
+
     flop_dense = 2.0 * S * C * C * 4          # 6 QKV + 2 out projections, per-stream rows
     flop_sdpa = 4.0 * H * S * S * D
     flop_block = flop_dense + flop_sdpa
@@ -181,7 +189,8 @@ def main():
 
     # ---------------- per-kernel timings (events on the launch stream) ----------------
     def time_kernel(fn, iters):
-        fn()
+        for _ in range(max(2, iters // 4)):
+            fn()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -202,20 +211,14 @@ def main():
         "dense_out_2x": time_kernel(k_out, it),
     }
     # the "palettized Dense alone" shape of the headline benchmark: M = 4608, 3072 -> 9216 (three weights) and 3072 -> 3072
-    x_all = f16((S, C))
-    y3 = [torch.empty((S, C), dtype=torch.float16, device=dev) for _ in range(3)]
     ms["dense_qkv_M4608_N9216"] = time_kernel(
         lambda: pkg.dense_multi(x_all, [w["x_q"], w["x_k"], w["x_v"]], [bias["x_q"], bias["x_k"], bias["x_v"]], outs=y3), it)
     ms["dense_out_M4608_N3072"] = time_kernel(
         lambda: pkg.dense_multi(x_all, [w["x_o"]], [bias["x_o"]], outs=[y3[0]]), it)
-    wf16 = pkg.QxTensor.from_f16(w["x_q"].dequantize())
     ms["dense_plainf16_M4608_N3072"] = time_kernel(
         lambda: pkg.dense_multi(x_all, [wf16], [bias["x_o"]], outs=[y3[0]]), it)
 
     # the op in front of the block's Dense layers: LayerNorm + adaLN modulation of the fp32 stream (HBM-bound)
-    x32 = torch.randn((S, C), dtype=torch.float32, device=dev)
-    ln_out = torch.empty((S, C), dtype=torch.float16, device=dev)
-    ln_scale, ln_shift = f16((C,), 0.2), f16((C,), 0.2)
     ms["layernorm_modulate"] = time_kernel(lambda: pkg.layernorm_modulate(x32, ln_scale, ln_shift, 1e-6, out=ln_out), max(it, 10))
 
     tf = lambda flop, t_ms: flop / (t_ms * 1e-3) / 1e12

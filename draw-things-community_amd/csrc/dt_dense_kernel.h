@@ -704,17 +704,31 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         }
       }
     };
-    RowIn cur;
-    if constexpr (FAST) fetch(0, cur);
-    for (int it = 0; it < WM / RPI; it++) {
+    // Trips go in groups of GRP: the rows a group needs from memory are requested one group ahead, before the
+    // previous group's stores (a load behind a store waits for it), so a trip does not wait a memory round trip.
+    constexpr int TRIPS = WM / RPI;
+    constexpr int GRP = (FAST && !POST) ? 4 : 1;
+    static_assert(TRIPS % GRP == 0, "trips per group");
+    RowIn cur[GRP];
+    if constexpr (FAST) {
+#pragma unroll
+      for (int j = 0; j < GRP; j++) fetch(j, cur[j]);
+    }
+    for (int it0 = 0; it0 < TRIPS; it0 += GRP) {
+      RowIn nxt[GRP];
+      if constexpr (FAST) {
+        if (it0 + GRP < TRIPS) {
+#pragma unroll
+          for (int j = 0; j < GRP; j++) fetch(it0 + GRP + j, nxt[j]);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < GRP; j++) {
+      const int it = it0 + j;
       const int t = it * RPI + rsub;
       const int64_t gm = m0 + wm * WM + t;
       const bool row_ok = FAST || gm < g.m;
       const int64_t gmc = row_ok ? gm : 0;
-      RowIn nxt;
-      if constexpr (FAST) {
-        if (it + 1 < WM / RPI) fetch(it + 1, nxt);  // before this row's stores: a load behind a store waits for it
-      }
       const uint4_t raw = *reinterpret_cast<const uint4_t*>(park + t * WN + ((c ^ (t & (CH - 1))) << 3));
       float v[8] = {lo16(raw[0]), hi16(raw[0]), lo16(raw[1]), hi16(raw[1]),
                     lo16(raw[2]), hi16(raw[2]), lo16(raw[3]), hi16(raw[3])};
@@ -733,7 +747,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         if (w.rot) {
           uint4_t rr;
           if constexpr (FAST) {
-            rr = cur.add;
+            rr = cur[j].add;
           } else {
             const uint16_t* rrow = w.rot + (w.rot_pos0 + gmc) * WN + 8 * c;
 #pragma unroll
@@ -754,8 +768,8 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
           if constexpr (FAST) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-              ad[2 * q] = lo16(cur.add[q]);
-              ad[2 * q + 1] = hi16(cur.add[q]);
+              ad[2 * q] = lo16(cur[j].add[q]);
+              ad[2 * q + 1] = hi16(cur[j].add[q]);
             }
           } else if (row_ok) {
 #pragma unroll
@@ -768,8 +782,8 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
           if constexpr (FAST) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-              ml[2 * q] = lo16(cur.mul[q]);
-              ml[2 * q + 1] = hi16(cur.mul[q]);
+              ml[2 * q] = lo16(cur[j].mul[q]);
+              ml[2 * q + 1] = hi16(cur[j].mul[q]);
             }
           } else if (row_ok) {
 #pragma unroll
@@ -781,8 +795,8 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
           if constexpr (FAST) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-              res[e] = cur.r0[e];
-              res[4 + e] = cur.r1[e];
+              res[e] = cur[j].r0[e];
+              res[4 + e] = cur[j].r1[e];
             }
           } else if (row_ok) {
 #pragma unroll
@@ -817,7 +831,11 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
             if (w.y) w.y[gmc * w.ldy + nn + e] = (uint16_t)(out[e >> 1] >> (16 * (e & 1)));
           }
       }
-      if constexpr (FAST) cur = nxt;
+      }
+      if constexpr (FAST) {
+#pragma unroll
+        for (int j = 0; j < GRP; j++) cur[j] = nxt[j];
+      }
     }
   };
   const bool aligned16 = (!w.y || (((w.ldy & 7) == 0) && (reinterpret_cast<uintptr_t>(w.y) & 15) == 0)) &&
