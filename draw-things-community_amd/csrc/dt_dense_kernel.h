@@ -137,8 +137,11 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// Two floats rounded to fp16 (round to nearest even) in one dword, as one packed conversion.
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
-  return (uint32_t)half_to_bits((half_t)a) | ((uint32_t)half_to_bits((half_t)b) << 16);
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
 }
 
 // 512 threads = 8 waves, two per SIMD, all eight running MFMAs on a (BN/2) x
