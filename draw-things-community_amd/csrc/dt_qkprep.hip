@@ -36,7 +36,7 @@ __device__ __forceinline__ uint32_t finish_pair(float a, float b, float inv, con
   return (uint32_t)half_to_bits((half_t)a) | ((uint32_t)half_to_bits((half_t)b) << 16);
 }
 
-// Per-head norm (or no norm): one wave per (b, s, h) row of D <= 128 elements,
+// Per-head norm (or no norm), any even D <= 128 and 4-byte alignment: one wave per (b, s, h) row,
 // lane p owns the complex pair (2p, 2p+1).
 __global__ void __launch_bounds__(256) qk_prep_head_kernel(const QkPrepArgs a) {
   const int lane = threadIdx.x & 63;
@@ -103,17 +103,172 @@ __global__ void __launch_bounds__(256) qk_prep_row_kernel(const QkPrepArgs a) {
   }
 }
 
+// ---- 16-byte forms ------------------------------------------------------------
+// The same arithmetic with every access a whole 16-byte chunk (8 elements = 4 complex pairs): used when the
+// head dimension is a multiple of 8 and every row, the table and the norm weight are 16-byte aligned.
+
+// normalise-rotate-scale the 8 elements of one chunk; g and r are the chunk's norm weights and table entries
+__device__ __forceinline__ uint4_t finish_chunk(const float (&x)[8], float inv, bool has_gamma, const uint4_t& g,
+                                                bool has_rot, const uint4_t& r, float post_scale) {
+  uint4_t out;
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    float a = x[2 * q], b = x[2 * q + 1];
+    if (has_gamma) {
+      a = round_h(a * inv * (float)bits_to_half((uint16_t)g[q]));
+      b = round_h(b * inv * (float)bits_to_half((uint16_t)(g[q] >> 16)));
+    }
+    if (has_rot) {
+      const float c = (float)bits_to_half((uint16_t)r[q]), sn = (float)bits_to_half((uint16_t)(r[q] >> 16));
+      const float na = round_h(a * c - b * sn);
+      const float nb = round_h(a * sn + b * c);
+      a = na;
+      b = nb;
+    }
+    if (post_scale != 1.0f) {
+      a = round_h(a * post_scale);
+      b = round_h(b * post_scale);
+    }
+    out[q] = (uint32_t)half_to_bits((half_t)a) | ((uint32_t)half_to_bits((half_t)b) << 16);
+  }
+  return out;
+}
+
+__device__ __forceinline__ void unpack_chunk(const uint4_t& v, float (&x)[8]) {
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    x[2 * q] = (float)bits_to_half((uint16_t)v[q]);
+    x[2 * q + 1] = (float)bits_to_half((uint16_t)(v[q] >> 16));
+  }
+}
+
+// Per-head norm (or none): LPR = D / 8 lanes (a power of two) per (b, s, h) row, 256 / LPR rows per pass of a
+// workgroup, kHeadPasses passes per thread with all their loads issued before the first use.
+constexpr int kHeadPasses = 4;
+template <int LPR>
+__global__ void __launch_bounds__(256) qk_prep_head16_kernel(const QkPrepArgs a) {
+  constexpr int RPP = 256 / LPR;  // rows per pass
+  const int c = threadIdx.x % LPR;
+  const int64_t rows = (int64_t)a.B * a.S * a.H;
+  const int64_t row0 = (int64_t)blockIdx.x * (RPP * kHeadPasses) + threadIdx.x / LPR;
+  uint4_t v[kHeadPasses], r[kHeadPasses] = {};
+  uint16_t* dst[kHeadPasses];
+  bool on[kHeadPasses];
+  uint4_t g = {0, 0, 0, 0};
+  if (a.gamma) g = *reinterpret_cast<const uint4_t*>(a.gamma + 8 * c);
+#pragma unroll
+  for (int i = 0; i < kHeadPasses; i++) {
+    const int64_t row = row0 + i * RPP;
+    on[i] = row < rows;
+    const int64_t rc = on[i] ? row : rows - 1;
+    const int h = (int)(rc % a.H);
+    const int64_t bs = rc / a.H;
+    const int64_t s = bs % a.S;
+    const int64_t b = bs / a.S;
+    v[i] = *reinterpret_cast<const uint4_t*>(a.src + b * a.src_sb + s * a.src_ss + h * a.src_sh + 8 * c);
+    dst[i] = a.dst + b * a.dst_sb + s * a.dst_ss + h * a.dst_sh + 8 * c;
+    if (a.rot) r[i] = *reinterpret_cast<const uint4_t*>(a.rot + (a.rot_pos0 + s) * a.D + 8 * c);
+  }
+#pragma unroll
+  for (int i = 0; i < kHeadPasses; i++) {
+    float x[8];
+    unpack_chunk(v[i], x);
+    float inv = 1.f;
+    if (a.gamma) {
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) ss += x[e] * x[e];
+#pragma unroll
+      for (int off = LPR / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      inv = 1.0f / sqrtf(ss / (float)a.D + a.eps);
+    }
+    const uint4_t out = finish_chunk(x, inv, a.gamma != nullptr, g, a.rot != nullptr, r[i], a.post_scale);
+    if (on[i]) *reinterpret_cast<uint4_t*>(dst[i]) = out;
+  }
+}
+
+// Whole-row norm over H * D <= 8192 elements: one wave per (b, s) row, the row held in registers between the
+// sum of squares and the output -- one read, one write.
+constexpr int kRowChunks = 16;  // 16-byte chunks per lane
+__global__ void __launch_bounds__(256) qk_prep_row16_kernel(const QkPrepArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t bs = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  if (bs >= (int64_t)a.B * a.S) return;
+  const int64_t s = bs % a.S;
+  const int64_t b = bs / a.S;
+  const int width = a.H * a.D;
+  const int nc = width / 8;  // chunks in the row
+  const uint16_t* src = a.src + b * a.src_sb + s * a.src_ss;
+  uint16_t* dst = a.dst + b * a.dst_sb + s * a.dst_ss;
+  uint4_t v[kRowChunks];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kRowChunks; i++) {
+    const int ch = lane + 64 * i;
+    v[i] = uint4_t{0, 0, 0, 0};
+    if (ch < nc) v[i] = *reinterpret_cast<const uint4_t*>(src + 8 * ch);
+  }
+#pragma unroll
+  for (int i = 0; i < kRowChunks; i++) {
+    float x[8];
+    unpack_chunk(v[i], x);
+#pragma unroll
+    for (int e = 0; e < 8; e++) ss += x[e] * x[e];
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)width + a.eps);
+  const uint16_t* rot_row = a.rot ? a.rot + (a.rot_pos0 + s) * a.D : nullptr;
+#pragma unroll
+  for (int i = 0; i < kRowChunks; i++) {
+    const int ch = lane + 64 * i;
+    if (ch < nc) {
+      float x[8];
+      unpack_chunk(v[i], x);
+      // the norm weight is indexed over the whole row, the table over the head dimension
+      const uint4_t g = *reinterpret_cast<const uint4_t*>(a.gamma + 8 * ch);
+      uint4_t r = {0, 0, 0, 0};
+      if (rot_row) r = *reinterpret_cast<const uint4_t*>(rot_row + (8 * ch) % a.D);
+      *reinterpret_cast<uint4_t*>(dst + 8 * ch) = finish_chunk(x, inv, true, g, rot_row != nullptr, r, a.post_scale);
+    }
+  }
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// every row of both views, the table and the norm weight can be accessed in 16-byte chunks
+static bool chunks_ok(const QkPrepArgs& a) {
+  return a.D % 8 == 0 && aligned16(a.src) && aligned16(a.dst) && a.src_sb % 8 == 0 && a.src_ss % 8 == 0 &&
+         a.src_sh % 8 == 0 && a.dst_sb % 8 == 0 && a.dst_ss % 8 == 0 && a.dst_sh % 8 == 0 &&
+         (!a.rot || aligned16(a.rot)) && (!a.gamma || aligned16(a.gamma));
+}
+
 dt_status qk_prep_launch(hipStream_t s, const QkPrepArgs& a) {
   if (a.B <= 0 || a.S <= 0 || a.H <= 0) return DT_OK;
   if (a.norm_per_head || !a.gamma) {
     int64_t rows = (int64_t)a.B * a.S * a.H;
+    const int lpr = a.D / 8;
+    if (chunks_ok(a) && (lpr == 16 || lpr == 8 || lpr == 4)) {
+      const int per_block = (256 / lpr) * kHeadPasses;
+      int64_t blocks = (rows + per_block - 1) / per_block;
+      if (blocks > 0x7fffffff) return DT_NO_KERNEL;
+      if (lpr == 16) hipLaunchKernelGGL(qk_prep_head16_kernel<16>, dim3((unsigned)blocks), dim3(256), 0, s, a);
+      else if (lpr == 8) hipLaunchKernelGGL(qk_prep_head16_kernel<8>, dim3((unsigned)blocks), dim3(256), 0, s, a);
+      else hipLaunchKernelGGL(qk_prep_head16_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, s, a);
+      return launch_status();
+    }
     int64_t blocks = (rows + 3) / 4;
     if (blocks > 0x7fffffff) return DT_NO_KERNEL;
     hipLaunchKernelGGL(qk_prep_head_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
   } else {
-    int64_t blocks = (int64_t)a.B * a.S;
-    if (blocks > 0x7fffffff) return DT_NO_KERNEL;
-    hipLaunchKernelGGL(qk_prep_row_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
+    const int64_t rows = (int64_t)a.B * a.S;
+    if (chunks_ok(a) && (int64_t)a.H * a.D <= 8 * 64 * kRowChunks) {
+      int64_t blocks = (rows + 3) / 4;
+      if (blocks > 0x7fffffff) return DT_NO_KERNEL;
+      hipLaunchKernelGGL(qk_prep_row16_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
+      return launch_status();
+    }
+    if (rows > 0x7fffffff) return DT_NO_KERNEL;
+    hipLaunchKernelGGL(qk_prep_row_kernel, dim3((unsigned)rows), dim3(256), 0, s, a);
   }
   return launch_status();
 }

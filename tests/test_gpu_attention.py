@@ -35,7 +35,7 @@ def ulp_close(got, want, ulps=1):
 
 # ------------------------------------------------------------------ K2
 
-@pytest.mark.parametrize("D,H", [(128, 24), (64, 8), (40, 8)])
+@pytest.mark.parametrize("D,H", [(128, 24), (64, 8), (40, 8), (32, 5)])
 def test_rmsnorm_per_head(dthip, oracle, torch_cuda, D, H):
     torch = torch_cuda
     rng = np.random.default_rng(D)
@@ -96,6 +96,25 @@ def test_norm_rope_scale_in_place_on_strided_view(dthip, oracle, torch_cuda):
     assert ulp_close(got[:, :, H * D:2 * H * D].reshape(B, S, H, D), want)
     # everything outside the view is untouched
     assert np.array_equal(got[:, :, :H * D], buf[:, :, :H * D]) and np.array_equal(got[:, :, 2 * H * D:], buf[:, :, 2 * H * D:])
+
+
+def test_norm_rope_rows_not_16_byte_aligned(dthip, oracle, torch_cuda):
+    """A view whose rows start 4 bytes off a 16-byte boundary takes the pair-per-lane kernel: same results."""
+    torch = torch_cuda
+    rng = np.random.default_rng(4)
+    B, S, H, D = 1, 41, 3, 128
+    buf = f16(rng.standard_normal((B, S, H * D + 2)))
+    g = f16(1 + 0.02 * rng.standard_normal(D))
+    rot = f16(dthip.Flux1RotaryPositionEmbedding(6, 6, 5, channels=D))
+    dev = to_dev(torch, buf)
+    view = dev[:, :, 2:].unflatten(2, (H, D))
+    print("norm rope unaligned", flush=True)
+    dthip.qk_norm_rope_(view, to_dev(torch, g), 1e-6, True, rot=to_dev(torch, rot), rot_pos0=0)
+    got = dev.cpu().numpy()
+    x = np.ascontiguousarray(buf[:, :, 2:]).reshape(B, S, H, D)
+    want = oracle.C.cmul(oracle.C.rmsnorm(x[0], g, 1e-6), rot[:S])
+    assert ulp_close(got[0, :, 2:].reshape(S, H, D), want)
+    assert np.array_equal(got[:, :, :2], buf[:, :, :2])
 
 
 # ------------------------------------------------------------------ K3
