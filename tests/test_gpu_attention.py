@@ -307,6 +307,37 @@ def test_sdpa_flux_full_size_sampled(dthip, oracle, torch_cuda):
     assert float((oc.float() - vc.float()).abs().max()) <= 2e-3
 
 
+def test_sdpa_flux_2048_full_size_sampled(dthip, oracle, torch_cuda):
+    """Long-sequence Flux shape (512 text + 16384 image tokens, 24 heads x 128), text and image as two segments:
+    sampled rows of two heads against the oracle, the constant-V property over the whole output, and the joint call
+    equal to the call on the concatenated tensors."""
+    torch = torch_cuda
+    rng = np.random.default_rng(22)
+    B, T, HW, H, D = 1, 512, 16384, 24, 128
+    S = T + HW
+    gen = torch.Generator(device="cuda").manual_seed(22)
+    qd = torch.randn((B, S, H, D), device="cuda", generator=gen).half()
+    kd = torch.randn((B, S, H, D), device="cuda", generator=gen).half()
+    vd = torch.randn((B, S, H, D), device="cuda", generator=gen).half()
+    scale = 1 / np.sqrt(D)
+    print("sdpa flux 2048 full size", flush=True)
+    got = dthip.sdpa_segments([qd[:, :T], qd[:, T:]], [kd[:, :T], kd[:, T:]], [vd[:, :T], vd[:, T:]], scale)
+    rows = np.sort(rng.choice(S, size=24, replace=False))
+    rows[0], rows[1], rows[-1] = 0, T, S - 1
+    rows = np.unique(rows)
+    rt = torch.from_numpy(rows).cuda()
+    for h in (0, 23):
+        want = oracle.C.sdpa(np.ascontiguousarray(qd[:, rt, h:h + 1].cpu().numpy()), np.ascontiguousarray(kd[:, :, h:h + 1].cpu().numpy()),
+                             np.ascontiguousarray(vd[:, :, h:h + 1].cpu().numpy()), scale)
+        mx, rr = oracle.err_stats(got[:, rt, h:h + 1].cpu().numpy(), want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (h, mx, rr)
+    whole = dthip.ScaledDotProductAttention(scale=scale)(qd, kd, vd)
+    assert torch.equal(got, whole)
+    vc = torch.from_numpy(f16(rng.standard_normal((1, 1, H, D)))).cuda().expand(B, S, H, D).contiguous()
+    oc = dthip.ScaledDotProductAttention(scale=scale)(qd, kd, vc)
+    assert float((oc.float() - vc.float()).abs().max()) <= 2e-3
+
+
 def test_sdpa_wan_full_size_sampled(dthip, oracle, torch_cuda):
     """The largest benchmark shape (1, 40 heads x 128, 32760 tokens; Q and K pre-scaled by D^-1/4 and scale 1, the
     `.scale1` convention of Models/Wan.swift:95-103): sampled rows of two heads against the oracle, the

@@ -555,6 +555,38 @@ def test_dense_post_bad_args(dthip, oracle, torch_cuda):
         dthip.LoRADense(64, dthip.LoRANetworkConfiguration(4, highPrecision=True))
 
 
+def test_dense_flux_2048_q4p_full_size_sampled(dthip, oracle, torch_cuda):
+    """Long-sequence Flux shape (M 16896, K 3072, three N 3072 q4p weights with 512-element blocks -- six palette
+    blocks per weight row -- in one launch): a sample of rows against the oracle, plus linearity Y(2x) == 2 Y(x)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(16)
+    M, K, N, q, nib = 16896, 3072, 3072, 4, 512
+    ws, packs, biases = [], [], []
+    for i in range(3):
+        w, p = make_weight(dthip, oracle, rng, N, K, q, nib)
+        ws.append(w)
+        packs.append(p)
+        biases.append((rng.standard_normal(N) * 0.02).astype(np.float16))
+    gen = torch.Generator(device="cuda").manual_seed(16)
+    xd = torch.randn((M, K), device="cuda", generator=gen).half()
+    print("dense flux 2048 q4p full size", flush=True)
+    outs = dthip.dense_multi(xd, ws, [to_dev(torch, b) for b in biases])
+    rows = np.sort(rng.choice(M, size=16, replace=False))
+    rows[0], rows[-1] = 0, M - 1
+    rt = torch.from_numpy(rows).cuda()
+    xr = np.ascontiguousarray(xd[rt].cpu().numpy())
+    for i in range(3):
+        want = oracle.C.dense_qx(xr, packs[i], q, nib, N, biases[i])
+        mx, rr = oracle.err_stats(outs[i][rt].cpu().numpy(), want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (i, mx, rr)
+    o1 = dthip.dense_multi(xd, ws, [None] * 3)
+    o2 = dthip.dense_multi(xd * 2, ws, [None] * 3)
+    for a, b in zip(o1, o2):
+        normal = a.abs() >= 2.0 ** -13
+        assert torch.equal((a * 2)[normal], b[normal])
+        assert float((a.float() * 2 - b.float()).abs().max()) <= 2.0 ** -23
+
+
 def test_dense_wan_full_size_sampled(dthip, oracle, torch_cuda):
     """The largest benchmark Dense (M 32760, 5120 -> 5120, q5p with 1024-element blocks: five palette blocks per weight
     row): a sample of rows against the oracle, plus linearity Y(2x) == 2 Y(x)."""
