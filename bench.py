@@ -148,7 +148,8 @@ def main():
         del src, dst
 
     # The step is three dependent launches; replayed as a HIP graph they go out without host gaps.  The graph is
-    # used only if its replays, with eager work in between, reproduce the eager outputs bit for bit.
+    # used only if its replays, with eager work in between, reproduce the eager outputs bit for bit, and only if
+    # a short trial shows it no slower than launching the three kernels one by one.
     run_step, launch_mode = step, "eager"
     if not args.no_graph:
         try:
@@ -172,7 +173,20 @@ def main():
                 step()  # eager work between replays
                 torch.cuda.synchronize()
             if ok:
-                run_step, launch_mode = graph.replay, "hip graph (3 kernels)"
+                # replays cost a little more per kernel than eager launches on some driver stacks: keep the quicker
+                def quick(fn, n=60):
+                    for _ in range(n):
+                        fn()
+                    torch.cuda.synchronize()
+                    t = time.perf_counter()
+                    for _ in range(n):
+                        fn()
+                    torch.cuda.synchronize()
+                    return time.perf_counter() - t
+                t_graph, t_eager = quick(graph.replay), quick(step)
+                t_graph, t_eager = min(t_graph, quick(graph.replay)), min(t_eager, quick(step))
+                if t_graph <= t_eager:
+                    run_step, launch_mode = graph.replay, "hip graph (3 kernels)"
         except Exception as e:  # capture not possible: stay eager
             print(f"graph capture failed, running eagerly: {e}", file=sys.stderr)
             torch.cuda.synchronize()
