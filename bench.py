@@ -25,6 +25,63 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {"dense_qkv": 4.715e8, "sdpa": 1.326e8}
 
 
+def other_configs(pkg, torch, np):
+    """Single operators of the benchmark configurations other than the Flux 1024 x 1024 block, at their full shapes:
+    events around a few launches each (weights stay hot in the memory-side cache), TFLOP/s from 2 M N K and
+    4 B H Sq Skv D."""
+    dev = "cuda"
+    rng = np.random.default_rng(1)
+
+    def timed(fn, n):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    def synth(N, K, q, nib):
+        count = N * K
+        pal = (rng.standard_normal(((count + nib - 1) // nib, 1 << q)) * 0.02).astype(np.float16)
+        idx = rng.integers(0, 1 << q, size=count, dtype=np.uint8)
+        return pkg.QxTensor.from_packed(pkg.pack_qx(q, nib, pal, idx), q, nib, (N, K))
+
+    out = {}
+
+    def record(name, flop, ms):
+        out[name] = {"ms": round(ms, 4), "tflops": round(flop / ms / 1e9, 1),
+                     "frac_f16_peak": round(flop / ms / 1e9 / PEAK_F16_TFLOPS, 4)}
+
+    def sdpa(name, B, Sq, Skv, H, D, n):
+        q = torch.randn(B, Sq, H, D, device=dev).half()
+        k = torch.randn(B, Skv, H, D, device=dev).half()
+        v = torch.randn_like(k)
+        o = torch.empty_like(q)
+        record(name, 4.0 * B * H * Sq * Skv * D, timed(lambda: pkg.sdpa_segments([q], [k], [v], 1 / np.sqrt(D), out=o), n))
+
+    def dense(name, M, K, Ns, codec, n):
+        qb, nb = pkg.CODEC[codec]
+        x = torch.randn(M, K, device=dev).half()
+        ws = [synth(N, K, qb, nb) for N in Ns]
+        outs = [torch.empty(M, N, device=dev, dtype=torch.float16) for N in Ns]
+        record(name, 2.0 * M * K * sum(Ns), timed(lambda: pkg.dense_multi(x, ws, [None] * len(ws), outs=outs), n))
+
+    sdpa("cfg1 SD1.5 self-attention B2 H8 D40 S4096", 2, 4096, 4096, 8, 40, 10)
+    sdpa("cfg1 SD1.5 cross-attention B2 H8 D40 Sq4096 Skv77", 2, 4096, 77, 8, 40, 10)
+    dense("cfg1 Dense q6p M8192 320->320", 8192, 320, [320], "q6p", 10)
+    dense("cfg2 Dense q8p M4608 3072->3x3072", 4608, 3072, [3072] * 3, "q8p", 10)
+    dense("cfg2 Dense q8p M4608 3072->3072", 4608, 3072, [3072], "q8p", 10)
+    sdpa("cfg4 Flux 2048^2 attention H24 D128 S16896", 1, 16896, 16896, 24, 128, 3)
+    dense("cfg4 Dense q4p M16896 3072->3x3072", 16896, 3072, [3072] * 3, "q4p", 3)
+    sdpa("cfg5 Wan self-attention H40 D128 S32760", 1, 32760, 32760, 40, 128, 2)
+    sdpa("cfg5 Wan cross-attention H40 D128 Sq32760 Skv512", 1, 32760, 512, 40, 128, 3)
+    dense("cfg5 Dense q5p M32760 5120->5120", 32760, 5120, [5120], "q5p", 2)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -38,6 +95,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--other-configs", action="store_true",
+                    help="also time the operators of the other benchmark configurations (SD 1.5, q8p Dense alone, "
+                         "Flux at 2048 x 2048 with q4p, Wan 14B with q5p) and add them to the JSON line as 'other_configs'")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1",
@@ -316,6 +376,8 @@ def main():
             "dense_gflops": round(flop_dense / t_dense / 1e9, 1), "sdpa_gflops": round(flop_sdpa / t_sdpa / 1e9, 1),
         }
 
+    other = other_configs(pkg, torch, np) if args.other_configs else None
+
     line = {
         "metric": "SDPA + palettized-GEMM TFLOP/s (% fp16 peak); ms/block, Flux 4608 tok q6p",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -327,6 +389,8 @@ def main():
         "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels,
         "block_ms_sum_of_kernels": round(dense_ms + ms["sdpa_S4608"], 4),
     }
+    if other is not None:
+        line["other_configs"] = other
     print(json.dumps(line))
 
 
