@@ -179,9 +179,16 @@ DT_EXPORT dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t
     a.o_sh = D;
     dt_status st = sdpa_launch(s, a);
     if (st != DT_OK) return st;
-    // unify-heads projection on the staged attention output, batch by batch
+    // unify-heads projection on the staged attention output: one Dense over all batches when the output's
+    // batches follow each other at the row stride, else batch by batch
     const int64_t HD = (int64_t)Hq * D;
     dt_qx_weight w{Wo, 16, 0, HD * HD};
+    if (B > 1 && o.stride_b == Sq * o.stride_s) {
+      const uint16_t* bias_arr[1] = {bo};
+      uint16_t* y_arr[1] = {static_cast<uint16_t*>(o.ptr)};
+      const int64_t ldy_arr[1] = {o.stride_s};
+      return dt_dense_qx_f16(stream, (int64_t)B * Sq, HD, ow, HD, &w, 1, bias_arr, y_arr, ldy_arr, 0);
+    }
     for (int b = 0; b < B; b++) {
       const uint16_t* bias_arr[1] = {bo};
       uint16_t* y_arr[1] = {static_cast<uint16_t*>(o.ptr) + b * o.stride_b};

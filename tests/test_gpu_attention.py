@@ -266,6 +266,12 @@ def test_sdpa_fused_output_projection(dthip, oracle, torch_cuda):
     want = oracle.C.dense(att, Wo, bo).reshape(B, Sq, H * D)
     mx, rr = oracle.err_stats(got, want)
     assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+    # an output whose batches are padded apart takes the projection batch by batch: same numbers
+    buf = torch.zeros((B, Sq + 3, H * D), dtype=torch.float16, device="cuda")
+    dthip.sdpa_segments([to_dev(torch, q)], [to_dev(torch, k)], [to_dev(torch, v)], 1 / np.sqrt(D),
+                        Wo=op.weight, bo=op.bias, out=buf[:, :Sq])
+    assert np.array_equal(buf[:, :Sq].cpu().numpy(), got)
+    assert float(buf[:, Sq:].abs().max()) == 0.0
 
 
 def test_sdpa_rejects_bad_arguments(dthip, torch_cuda):
