@@ -27,15 +27,26 @@ MEASURED_TRAFFIC_BYTES = {"dense_qkv": 4.715e8, "sdpa": 1.326e8}
 
 def other_configs(pkg, torch, np):
     """Single operators of the benchmark configurations other than the Flux 1024 x 1024 block, at their full shapes:
-    events around a few launches each (weights stay hot in the memory-side cache), TFLOP/s from 2 M N K and
-    4 B H Sq Skv D."""
+    events around ~100 ms of back-to-back launches each, after ~50 ms of warm-up (weights stay hot in the
+    memory-side cache), TFLOP/s from 2 M N K and 4 B H Sq Skv D."""
     dev = "cuda"
     rng = np.random.default_rng(1)
 
     def timed(fn, n):
+        # at least ~50 ms of warm-up and ~100 ms of timed work, so that short kernels are measured at the
+        # sustained clock like the step above
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         fn()
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        torch.cuda.synchronize()
+        once = max(e0.elapsed_time(e1), 1e-3)
+        for _ in range(min(2000, int(50.0 / once))):
+            fn()
+        n = max(n, min(4000, int(100.0 / once)))
+        torch.cuda.synchronize()
         e0.record()
         for _ in range(n):
             fn()
