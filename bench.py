@@ -22,7 +22,7 @@ PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
 # counters read for a 256 MiB device copy (x2.00 and x1.00); the summary is profiles/bench_flux_block_counters.txt
-MEASURED_TRAFFIC_BYTES = {"dense_qkv": 4.715e8, "sdpa": 1.326e8}
+MEASURED_TRAFFIC_BYTES = {"dense_qkv": 3.750e8, "sdpa": 1.326e8}
 
 
 def other_configs(pkg, torch, np):

@@ -193,10 +193,11 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const int lt = tid & 255;
   const int wn = wave & 1, wm = ((wave >> 1) & 1) | ((wave >> 2) << 1);  // waves w and w+4 share a SIMD and take different m slices
 
-  // Tile order: bands of 8 token tiles; inside a band feature tiles outermost,
+  // Tile order: bands of 4 token tiles; inside a band feature tiles outermost,
   // token tiles innermost.  Workgroups are dealt round-robin to the 8 XCDs;
   // giving each XCD a contiguous run of that order makes the workgroups that
-  // run together on an XCD cover a compact 2-D block of tiles (8 x 4 at 32 CUs),
+  // run together on an XCD cover a compact 2-D block of tiles (4 token tiles x 8
+  // feature tiles at 32 CUs: an X slice is 16 KB per K-tile, a packed W slice 4-8 KB),
   // so every X and W panel slice is fetched into that XCD's L2 once per block
   // instead of once per tile column.
   const int total = a.total_tiles;
@@ -213,7 +214,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   bid -= g.tile_begin;
   int tm, tn;
   {
-    constexpr int GM = 8;
+    constexpr int GM = 4;
     const int band_tiles = GM * g.tiles_n;
     const int band = bid / band_tiles;
     const int in_band = bid - band * band_tiles;
