@@ -60,7 +60,8 @@ __device__ __forceinline__ float act_gelu_tanh(float x) {
 __device__ __forceinline__ float act_swish(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
 }
-__device__ __forceinline__ float act_gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f)); }
+// 1 + erf(z) = erfc(-z): no cancellation for large negative x
+__device__ __forceinline__ float act_gelu_erf(float x) { return 0.5f * x * erfcf(x * -0.7071067811865476f); }
 __device__ __forceinline__ float post_value(float v, float scale, bool has_add, float add, bool has_mul, float mul, int act,
                                             bool has_gate, float gate) {
   if (scale != 1.0f) v = (float)(half_t)(v * scale);

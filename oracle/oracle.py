@@ -341,16 +341,19 @@ def synth_qx_weight(rng, N, K, qbits, nib, std=0.02):
 
 
 # ---------------------------------------------------------------------------
-# Elementwise tails of the feed-forward / residual paths (numpy; fp16 in, fp16 out, computed in float32 as the
-# reference's elementwise ops do).  Pinned in tests/test_oracle_ops.py by float64 closed forms (erf-GELU bound,
+# Elementwise tails of the feed-forward / residual paths (numpy; fp16 in, fp16 out; the activations are the
+# mathematical functions, evaluated in float64 and rounded once).  Pinned in tests/test_oracle_ops.py by float64 closed forms (erf-GELU bound,
 # gelu(x) - gelu(-x) = x, limits, sigmoid identity) and exact small cases of the residual update.  GELU(approximate: .tanh): Models/Flux1.swift:133-135; swish: :122-123;
 # gated residual x + (y .* gate).to(of: x): :246-250, 275-283.
 # ---------------------------------------------------------------------------
 
 def np_gelu_tanh16(y16: np.ndarray) -> np.ndarray:
-    x = y16.astype(np.float32)
-    u = np.float32(0.7978845608028654) * (x + np.float32(0.044715) * x * x * x)
-    return (np.float32(0.5) * x * (np.float32(1) + np.tanh(u))).astype(np.float16)
+    """GELU(approximate: .tanh), 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))), evaluated in float64 and rounded
+    once: the function itself.  (Evaluated in float32 as written, `1 + tanh(u)` cancels for x < -3: over all fp16
+    inputs that form is up to 3 fp16 ulps -- 1.5e-7 in absolute terms -- off this one, on outputs below 2^-10.)"""
+    x = y16.astype(np.float64)
+    u = 0.7978845608028654 * (x + 0.044715 * x * x * x)
+    return (0.5 * x * (1.0 + np.tanh(u))).astype(np.float32).astype(np.float16)
 
 
 def np_gelu_erf16(y16: np.ndarray) -> np.ndarray:
@@ -381,8 +384,10 @@ def np_layernorm16(x16: np.ndarray, gamma16=None, beta16=None, eps: float = 1e-5
 
 
 def np_swish16(y16: np.ndarray) -> np.ndarray:
-    x = y16.astype(np.float32)
-    return (x / (np.float32(1) + np.exp(-x))).astype(np.float16)
+    """x sigmoid(x) in float64, rounded once."""
+    x = y16.astype(np.float64)
+    with np.errstate(over="ignore"):
+        return (x / (1.0 + np.exp(-x))).astype(np.float32).astype(np.float16)
 
 
 def np_layernorm_modulate16(x32: np.ndarray, scale=None, shift=None, eps: float = 1e-6, mod: str = "f16") -> np.ndarray:

@@ -610,3 +610,34 @@ def test_dense_wan_full_size_sampled(dthip, oracle, torch_cuda):
     normal = a.abs() >= 2.0 ** -13
     assert torch.equal((a * 2)[normal], b[normal])
     assert float((a.float() * 2 - b.float()).abs().max()) <= 2.0 ** -23
+
+
+def test_dense_post_activations_over_every_fp16_input(dthip, oracle, torch_cuda):
+    """Every finite fp16 value goes through a Dense with an identity weight (one non-zero term per output: y == x)
+    and then through each activation of the elementwise tail: the result is within one fp16 ulp of the function
+    evaluated in float64 and rounded once, over the whole input domain (tiny outputs for x < -3 included, where
+    1 + tanh(u) and 1 + erf(z) would cancel)."""
+    torch = torch_cuda
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    x16 = bits.view(np.float16).copy()
+    x16[~np.isfinite(x16)] = 0
+    x16 = x16.reshape(1024, 64)
+    w = dthip.QxTensor.from_f16(np.eye(64, dtype=np.float16))
+    xd = to_dev(torch, x16)
+    print("dense post activations, whole fp16 domain", flush=True)
+    plain = dthip.dense_multi(xd, [w], [None])[0].cpu().numpy()
+    assert np.array_equal(plain, x16)  # (as values: -0 comes back as +0)
+
+    def ulps(a, b):
+        ai, bi = a.view(np.int16).astype(np.int32), b.view(np.int16).astype(np.int32)
+        ai = np.where(ai < 0, -32768 - ai, ai)
+        bi = np.where(bi < 0, -32768 - bi, bi)
+        return np.abs(ai - bi)
+
+    for act, fn in ((dthip.ACT_GELU_TANH, oracle.np_gelu_tanh16), (dthip.ACT_SWISH, oracle.np_swish16),
+                    (dthip.ACT_GELU_ERF, oracle.np_gelu_erf16)):
+        got = dthip.dense_post(xd, [w], [None], [dthip.DensePost(act)])[0].cpu().numpy()
+        want = fn(x16)
+        assert np.array_equal(np.isfinite(got), np.isfinite(want)), act
+        ok = np.isfinite(want)
+        assert int(ulps(got, want)[ok].max()) <= 1, (act, int(ulps(got, want)[ok].max()))
