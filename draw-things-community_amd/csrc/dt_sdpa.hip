@@ -281,10 +281,13 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       for (int v = 0; v < 16; v++) sacc[kb][v] = 0.f;
     // K fragments are read two k-steps (4 reads) ahead of the MFMAs that use them
     half8_t kf[2][4];
+    // (a k-step that lies wholly in the zero padding of a short head -- the fourth at D = 40 -- is left out)
+    auto live = [&](int ks) __attribute__((always_inline)) { return DP != 64 || ks * 16 < D; };
     auto read_k = [&](int buf, int g) __attribute__((always_inline)) {
 #pragma unroll
       for (int u = 0; u < 4; u++)
-        kf[buf][u] = *reinterpret_cast<const half8_t*>(kt + (u & 1) * 32 * ROWB + k_rd[2 * g + (u >> 1)]);
+        if (live(2 * g + (u >> 1)))
+          kf[buf][u] = *reinterpret_cast<const half8_t*>(kt + (u & 1) * 32 * ROWB + k_rd[2 * g + (u >> 1)]);
     };
     read_k(0, 0);
 #pragma unroll
@@ -294,7 +297,8 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int u = 0; u < 4; u++)
-        sacc[u & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[g & 1][u], qf[2 * g + (u >> 1)], sacc[u & 1], 0, 0, 0);
+        if (live(2 * g + (u >> 1)))
+          sacc[u & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[g & 1][u], qf[2 * g + (u >> 1)], sacc[u & 1], 0, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
