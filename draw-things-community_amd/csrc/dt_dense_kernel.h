@@ -694,8 +694,11 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     float4_t r0, r1;
   };
   // FAST: the wave's slice lies inside the matrix and every row meets the vector alignment
-  auto walk = [&](auto fast_tag) {
+  // ACT: the activation when it is known where the loop is instantiated (the fast form is instantiated once
+  // per activation, so that its body holds one activation's code and no branches), or -1 = read it per element
+  auto walk = [&](auto fast_tag, auto act_tag) {
     constexpr bool FAST = decltype(fast_tag)::value;
+    constexpr int ACT = decltype(act_tag)::value;
     auto fetch = [&](int it, RowIn& in) {
       const int t = it * RPI + rsub;
       const int64_t gm = m0 + wm * WM + t;
@@ -809,12 +812,43 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
               if (nn + e < w.n) res[e] = w.res[gmc * w.ld_res + nn + e];
           }
         }
+        // post_value's steps, each over the row's 8 values under one uniform test (a step that is off costs a
+        // branch, not eight selects)
+        const auto rh = [](float x) { return (float)(half_t)x; };
+        if (w.scale != 1.0f) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-          v[e] = post_value(v[e], w.scale, w.add != nullptr, ad[e], w.mul != nullptr, ml[e], w.act, w.gate != nullptr, gt[e]);
-          float pr = w.gate32 ? v[e] * gt[e] : v[e];  // the fp32 gate's product is its own op: rounded before the addition
-          asm volatile("" : "+v"(pr));
-          res[e] += pr;
+          for (int e = 0; e < 8; e++) v[e] = rh(v[e] * w.scale);
+        }
+        if (w.add) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(v[e] + ad[e]);
+        }
+        if (w.mul) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(v[e] * ml[e]);
+        }
+        const int act = ACT >= 0 ? ACT : w.act;
+        if (act == DT_ACT_GELU_TANH) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(act_gelu_tanh(v[e]));
+        } else if (act == DT_ACT_SWISH) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(act_swish(v[e]));
+        } else if (act == DT_ACT_GELU_ERF) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(act_gelu_erf(v[e]));
+        }
+        if (w.gate) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(v[e] * gt[e]);
+        }
+        if (w.res) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            float pr = w.gate32 ? v[e] * gt[e] : v[e];  // the fp32 gate's product is its own op: rounded before the addition
+            asm volatile("" : "+v"(pr));
+            res[e] += pr;
+          }
         }
       }
       const uint4_t out = {pack_h2(v[0], v[1]), pack_h2(v[2], v[3]), pack_h2(v[4], v[5]), pack_h2(v[6], v[7])};
@@ -848,8 +882,20 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
                          (!POST || ((!w.add || (((w.ld_add & 7) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 15) == 0)) &&
                                     (!w.mul || (((w.ld_mul & 7) == 0) && (reinterpret_cast<uintptr_t>(w.mul) & 15) == 0)) &&
                                     (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0))));
-  if (aligned16 && nw + WN <= w.n && m0 + wm * WM + WM <= g.m) walk(std::true_type{});
-  else walk(std::false_type{});
+  if (aligned16 && nw + WN <= w.n && m0 + wm * WM + WM <= g.m) {
+    if constexpr (POST) {
+      switch (w.act) {
+        case DT_ACT_GELU_TANH: walk(std::true_type{}, std::integral_constant<int, DT_ACT_GELU_TANH>{}); break;
+        case DT_ACT_SWISH: walk(std::true_type{}, std::integral_constant<int, DT_ACT_SWISH>{}); break;
+        case DT_ACT_GELU_ERF: walk(std::true_type{}, std::integral_constant<int, DT_ACT_GELU_ERF>{}); break;
+        default: walk(std::true_type{}, std::integral_constant<int, DT_ACT_NONE>{}); break;
+      }
+    } else {
+      walk(std::true_type{}, std::integral_constant<int, DT_ACT_NONE>{});
+    }
+  } else {
+    walk(std::false_type{}, std::integral_constant<int, -1>{});
+  }
 }
 
 
