@@ -125,3 +125,100 @@ def test_norm_rope_random_shapes(dthip, oracle, torch_cuda):
             tol = np.repeat(np.maximum(mag * 2.0 ** -10, 2.0 ** -14), 2, axis=-1)
             diff = np.abs(got[b, :, off:].reshape(S, H, D).astype(np.float32) - wf)
             assert (diff <= tol).all(), (i, float((diff / tol).max()))
+
+
+def _weight(dthip, oracle, rng, N, K, q, nib):
+    if q == 16:
+        return dthip.QxTensor.from_f16(f16(rng.standard_normal((N, K)) * 0.05))
+    packed, _, _ = oracle.synth_qx_weight(rng, N, K, q, nib, 0.05)
+    return dthip.QxTensor.from_packed(packed, q, nib, (N, K))
+
+
+def _ulps(a, b):
+    ai, bi = a.view(np.int16).astype(np.int32), b.view(np.int16).astype(np.int32)
+    ai = np.where(ai < 0, -32768 - ai, ai)
+    bi = np.where(bi < 0, -32768 - bi, bi)
+    return int(np.abs(ai - bi).max())
+
+
+def test_dense_tails_random_shapes(dthip, oracle, torch_cuda):
+    """Activation, gate and fp32 residual in the Dense epilogue on random shapes, against numpy on the device's own
+    plain Dense result: the fp16 output within one ulp per rounded step that follows an activation (exact without
+    one), the residual stream within the rounding of its addition."""
+    torch = torch_cuda
+    rng = np.random.default_rng(104)
+    acts = {dthip.ACT_NONE: lambda y: y, dthip.ACT_GELU_TANH: oracle.np_gelu_tanh16, dthip.ACT_SWISH: oracle.np_swish16,
+            dthip.ACT_GELU_ERF: oracle.np_gelu_erf16}
+    for i in range(N_CASES):
+        q = int(rng.choice([4, 5, 6, 8, 16]))
+        nib = int(rng.choice([64, 512, 1024, 4096, 16384]))
+        K = int(rng.choice([64, 128, 192, 320, 512, 1024]))
+        M = int(rng.choice([1, 64, 127, 129, 256, 300, 1024, 1100, 2049]))
+        N = int(rng.choice([8, 72, 128, 256, 384, 520]))
+        act = int(rng.choice(list(acts)))
+        use_gate, use_res = rng.random() < 0.5, rng.random() < 0.6
+        keep = (rng.random() < 0.7) or not use_res
+        print("dense tail", i, q, nib, M, K, N, act, use_gate, use_res, keep, flush=True)
+        w = _weight(dthip, oracle, rng, N, K, q, nib)
+        xd = to_dev(torch, f16(rng.standard_normal((M, K))))
+        bd = to_dev(torch, f16(rng.standard_normal(N) * 0.1))
+        gate = f16(1 + 0.3 * rng.standard_normal(N))
+        res0 = rng.standard_normal((M, N)).astype(np.float32)
+        plain = dthip.dense_multi(xd, [w], [bd])[0].cpu().numpy()
+        res = torch.from_numpy(res0.copy()).cuda() if use_res else None
+        o = dthip.dense_post(xd, [w], [bd], [dthip.DensePost(act, gate=to_dev(torch, gate) if use_gate else None,
+                                                              residual=res, keep_output=keep)])[0]
+        y = acts[act](plain)
+        if use_gate:
+            y = (y.astype(np.float32) * gate.astype(np.float32)[None, :]).astype(np.float16)
+        if keep:
+            allowed = 0 if act == dthip.ACT_NONE else (2 if use_gate else 1)
+            assert _ulps(o.cpu().numpy(), y) <= allowed, i
+        else:
+            assert o is None
+        if use_res:
+            err = np.max(np.abs(res.cpu().numpy() - (res0 + y.astype(np.float32))))
+            assert err <= 2.0 ** -9 * max(1.0, float(np.abs(y.astype(np.float32)).max())), (i, err)
+
+
+def test_dense_fused_heads_random_shapes(dthip, oracle, torch_cuda):
+    """Per-head RMSNorm + RoPE behind the projection (in the GEMM epilogue for 128-wide heads, as a pass after it
+    otherwise) on random shapes, against the oracle's norm and rotation of the device's own plain Dense result.
+    Two fp16 ulps of a pair's magnitude: one for a rounding of the normalised value that falls the other way (the
+    sums of squares are added in another order), which the rotation then carries into both components."""
+    torch = torch_cuda
+    rng = np.random.default_rng(105)
+    for i in range(N_CASES):
+        q = int(rng.choice([4, 5, 6, 8, 16]))
+        nib = int(rng.choice([64, 512, 1024, 4096, 16384]))
+        K = int(rng.choice([64, 128, 192, 320, 512, 1024]))
+        M = int(rng.choice([1, 64, 127, 129, 256, 300, 1024, 1100, 2049]))
+        hd = int(rng.choice([128, 128, 64, 40]))
+        H = int(rng.choice([1, 2, 3]))
+        N, pos0 = H * hd, int(rng.choice([0, 5]))
+        print("dense heads", i, q, nib, M, K, hd, H, flush=True)
+        ws = [_weight(dthip, oracle, rng, N, K, q, nib) for _ in range(3)]
+        bs = [to_dev(torch, f16(rng.standard_normal(N) * 0.05)) for _ in range(3)]
+        gs = [f16(1 + 0.05 * rng.standard_normal(hd)) for _ in range(2)]
+        th = rng.uniform(-3, 3, size=(pos0 + M, hd // 2))
+        rot = np.empty((pos0 + M, hd), np.float16)
+        rot[:, 0::2], rot[:, 1::2] = np.cos(th), np.sin(th)
+        rd = to_dev(torch, rot)
+        use = [(True, True), (rng.random() < 0.7, rng.random() < 0.8)]
+        epi = [dthip.HeadEpilogue(to_dev(torch, gs[j]) if use[j][0] else None, rd if use[j][1] else None, pos0, 1e-6, hd)
+               for j in range(2)] + [None]
+        xd = to_dev(torch, f16(rng.standard_normal((M, K))))
+        outs = dthip.dense_multi(xd, ws, bs, epilogues=epi)
+        plain = dthip.dense_multi(xd, ws, bs)
+        assert torch.equal(outs[2], plain[2])
+        for j in range(2):
+            y = plain[j].cpu().numpy().reshape(M, H, hd)
+            if use[j][0]:
+                y = oracle.C.rmsnorm(y, gs[j], 1e-6)
+            if use[j][1]:
+                y = oracle.C.cmul(y, rot[pos0:pos0 + M])
+            wf = y.astype(np.float32)
+            mag = np.sqrt(wf[..., 0::2] ** 2 + wf[..., 1::2] ** 2)
+            tol = np.repeat(np.maximum(mag * 2.0 ** -9, 2.0 ** -14), 2, axis=-1)
+            diff = np.abs(outs[j].cpu().numpy().reshape(M, H, hd).astype(np.float32) - wf)
+            assert (diff <= tol).all(), (i, j, float((diff / tol).max()))
