@@ -695,7 +695,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   };
   // FAST: the wave's slice lies inside the matrix and every row meets the vector alignment
   // ACT: the activation when it is known where the loop is instantiated (the fast form is instantiated once
-  // per activation, so that its body holds one activation's code and no branches), or -1 = read it per element
+  // per activation, so that its body holds one activation's code), or -1 = taken from the arguments at run time
   auto walk = [&](auto fast_tag, auto act_tag) {
     constexpr bool FAST = decltype(fast_tag)::value;
     constexpr int ACT = decltype(act_tag)::value;
