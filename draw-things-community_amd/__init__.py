@@ -487,8 +487,8 @@ class LoRADense:
     """LoRADense(count:configuration:noBias:flags:name:) -- dense(x) + up(scale * down(x)) with the palettized base
     left packed and the fp16 low-rank pair applied beside it (Models/LoRA.swift:85-142; running the LoRA separately
     is the preferred mode for quantized models, Models/UNetProtocol.swift:696-697).  Three launches of the Dense
-    kernel: down (with the scale in its epilogue), up, then the base projection whose epilogue adds the branch; every
-    intermediate is rounded to fp16 as the reference's separate ops round.  `highPrecision` (an fp32 down
+    kernel: down (with the scale in its epilogue) beside the base projection, then up, whose epilogue adds the base
+    projection's result; every intermediate is rounded to fp16 as the reference's separate ops round.  `highPrecision` (an fp32 down
     projection) is not provided by the library."""
 
     def __init__(self, count: int, configuration: LoRANetworkConfiguration, noBias: bool = False, flags: int = 0,
@@ -530,11 +530,35 @@ class LoRADense:
         if self.down.shape[0] != self.configuration.rank or self.up.shape != (self.count, self.configuration.rank):
             raise ValueError(f"LoRADense {self.name!r}: down / up shapes do not match rank and count")
         dn, up = self._padded()
-        down = dense_post(x, [dn], [None], [DensePost(scale=self.configuration.scale)], stream=stream)[0]
-        branch = dense_multi(down, [up], [None], stream=stream)[0]
         p = post or DensePost()
-        tail = DensePost(p.activation, p.gate, p.residual, p.keep_output, addend=branch.reshape(-1, self.count))
-        return dense_post(x, [self.weight], [b], [tail], flags=self.flags, stream=stream)[0]
+        if p.scale != 1.0 or p.addend is not None or p.multiplicand is not None:
+            raise ValueError(f"LoRADense {self.name!r}: the tail may carry an activation, a gate and a residual only")
+        # The down projection is a few dozen workgroups that wait on memory; the base projection does not depend on
+        # it.  They go out side by side on two streams, and the up projection, whose epilogue adds the base
+        # projection's result and then runs the tail, follows both.  (fp16(base) + fp16(branch) rounds the same
+        # whichever of the two is the addend.)
+        torch = _torch()
+        main = stream if stream is not None else torch.cuda.current_stream(x.device)
+        side = _side_stream(x.device)
+        side.wait_stream(main)
+        down = dense_post(x, [dn], [None], [DensePost(scale=self.configuration.scale)], stream=side)[0]
+        base = dense_multi(x, [self.weight], [b], flags=self.flags, stream=main)[0]
+        main.wait_stream(side)  # every use of x and `down` on the side stream is ordered before what follows on `main`
+        tail = DensePost(p.activation, p.gate, p.residual, p.keep_output, addend=base.reshape(-1, self.count))
+        out = dense_post(down, [up], [None], [tail], stream=main)[0]
+        return None if out is None else out.reshape(*x.shape[:-1], self.count)
+
+
+_SIDE_STREAMS = {}
+
+
+def _side_stream(device):
+    """One extra stream per device (default priority) for work that may run beside the caller's stream."""
+    torch = _torch()
+    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+    if key not in _SIDE_STREAMS:
+        _SIDE_STREAMS[key] = torch.cuda.Stream(device=key)
+    return _SIDE_STREAMS[key]
 
 
 def _view4(t) -> _View4:

@@ -440,6 +440,23 @@ def test_lora_dense(dthip, oracle, torch_cuda, M, N, K, q, nib, rank, scale):
     o = dthip.dense_post(xd, [w], [bd], [dthip.DensePost(dthip.ACT_GELU_TANH, addend=wide[:, 4:4 + N])])[0]
     g = layer(xd, post=dthip.DensePost(dthip.ACT_GELU_TANH))
     assert torch.equal(o, g)
+    # the layer forks its down projection onto a second stream and joins it again: as a captured graph too
+    cs = torch.cuda.Stream()
+    cs.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(cs):
+        layer(xd)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=cs):
+            captured = layer(xd)
+        for _ in range(2):
+            captured.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(captured.cpu().numpy().view(np.uint16), out.view(np.uint16))
+            layer(xd)  # eager work between the replays
+            torch.cuda.synchronize()
+    torch.cuda.current_stream().wait_stream(cs)
     # one fp16 ulp, or 2^-19 where GELU's 1 + tanh cancels (inputs below -3: results of 1e-4 and less)
     got16, want16 = o.cpu().numpy(), oracle.np_gelu_tanh16(out)
     tol = np.maximum(np.spacing(np.abs(want16)).astype(np.float32), np.float32(2.0 ** -19))
