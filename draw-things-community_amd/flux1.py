@@ -17,7 +17,7 @@ from typing import Dict, Optional, Sequence
 
 import numpy as np
 
-from . import (ACT_GELU_TANH, DensePost, HeadEpilogue, QxTensor, dense_grouped, dense_multi, dense_post,
+from . import (ACT_GELU_TANH, DensePost, HeadEpilogue, QxTensor, _side_stream, dense_grouped, dense_multi, dense_post,
                layernorm_modulate, sdpa_segments, _torch)
 
 DENSE_NAMES = ("c_q", "c_k", "c_v", "x_q", "x_k", "x_v", "c_o", "x_o", "c_linear1", "c_out_proj", "x_linear1",
@@ -61,11 +61,23 @@ class JointTransformerBlock:
         W, Bv, G = self.weight, self.bias, self.norm
         buf = self._alloc(x.device)
         qkv, att, cn, xn = buf["qkv"], buf["att"], buf["cn"], buf["xn"]
-        c_res = context.reshape(t, C).clone()
-        x_res = x.reshape(hw, C).clone()
+        # The block returns new streams, so the residual epilogues accumulate into copies.  The copies are made on a
+        # second stream beside the attention half's launches, which read the originals; the context stream's
+        # LayerNorm launches (short, independent of the image stream's) go there too.
+        main = stream if stream is not None else torch.cuda.current_stream(x.device)
+        side = _side_stream(x.device)
+        c_in, x_in = context.reshape(t, C), x.reshape(hw, C)
+        c_res, x_res = torch.empty_like(c_in), torch.empty_like(x_in)
+        side.wait_stream(main)
         # attention half
-        layernorm_modulate(c_res, contextChunks[1], contextChunks[0], 1e-6, out=cn, stream=stream)
-        layernorm_modulate(x_res, xChunks[1], xChunks[0], 1e-6, out=xn, stream=stream)
+        layernorm_modulate(c_in, contextChunks[1], contextChunks[0], 1e-6, out=cn, stream=side)
+        context_normed = side.record_event()
+        with torch.cuda.stream(side):
+            c_res.copy_(c_in)
+            x_res.copy_(x_in)
+        copied = side.record_event()
+        layernorm_modulate(x_in, xChunks[1], xChunks[0], 1e-6, out=xn, stream=main)
+        main.wait_event(context_normed)
         qkv2 = qkv.view(S, 3 * C)
         views = lambda lo, hi: [qkv2[lo:hi, i * C:(i + 1) * C] for i in range(3)]
         epi = lambda q, kk, pos: [HeadEpilogue(G[q], rot, pos, 1e-6, k), HeadEpilogue(G[kk], rot, pos, 1e-6, k), None]
@@ -77,14 +89,17 @@ class JointTransformerBlock:
         sdpa_segments([qkv[:, 0].unsqueeze(0)], [qkv[:, 1].unsqueeze(0)], [qkv[:, 2].unsqueeze(0)],
                       1.0 / float(np.sqrt(k)), out=att, stream=stream)
         att2 = att.view(S, C)
+        main.wait_event(copied)
         tail = lambda gate, res: [DensePost(gate=gate, residual=res, keep_output=False)]
         dense_grouped([
             dict(x=att2[t:], weights=[W["x_o"]], biases=[Bv["x_o"]], posts=tail(xChunks[2], x_res)),
             dict(x=att2[:t], weights=[W["c_o"]], biases=[Bv["c_o"]], posts=tail(contextChunks[2], c_res))],
             stream=stream)
         # feed-forward half
-        layernorm_modulate(c_res, contextChunks[4], contextChunks[3], 1e-6, out=cn, stream=stream)
-        layernorm_modulate(x_res, xChunks[4], xChunks[3], 1e-6, out=xn, stream=stream)
+        side.wait_stream(main)
+        layernorm_modulate(c_res, contextChunks[4], contextChunks[3], 1e-6, out=cn, stream=side)
+        layernorm_modulate(x_res, xChunks[4], xChunks[3], 1e-6, out=xn, stream=main)
+        main.wait_stream(side)
         gelu = [DensePost(ACT_GELU_TANH)]
         dense_grouped([
             dict(x=xn, weights=[W["x_linear1"]], biases=[Bv["x_linear1"]], outs=[buf["xh"]], posts=gelu),
