@@ -138,8 +138,15 @@ class SingleTransformerBlock:
         if tuple(x.shape[-2:]) != (S, C) or len(xChunks) != 3:
             raise ValueError("x / xChunks do not match the block")
         W, Bv, G = self.weight, self.bias, self.norm
-        res = x.reshape(S, C).clone()
-        xn = layernorm_modulate(res, xChunks[1], xChunks[0], 1e-6, stream=stream)
+        # the copy that the last epilogue accumulates into is made on a second stream, beside the launches below
+        main = stream if stream is not None else torch.cuda.current_stream(x.device)
+        side = _side_stream(x.device)
+        x_in = x.reshape(S, C)
+        res = torch.empty_like(x_in)
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            res.copy_(x_in)
+        xn = layernorm_modulate(x_in, xChunks[1], xChunks[0], 1e-6, stream=stream)
         qkv = torch.empty((S, 3, h, k), dtype=torch.float16, device=x.device)
         qkv2 = qkv.view(S, 3 * C)
         dense_multi(xn, [W["x_q"], W["x_k"], W["x_v"]], [Bv["x_q"], Bv["x_k"], Bv["x_v"]],
@@ -150,6 +157,7 @@ class SingleTransformerBlock:
                             1.0 / float(np.sqrt(k)), stream=stream)
         hid = dense_post(xn, [W["x_linear1"]], [Bv["x_linear1"]], [DensePost(ACT_GELU_TANH)], stream=stream)[0]
         heads = dense_multi(att.view(S, C), [W["x_o"]], [None], stream=stream)[0]
+        main.wait_stream(side)
         dense_post(hid, [W["x_out_proj"]], [Bv["x_out_proj"]],
                    [DensePost(gate=xChunks[2], residual=res, keep_output=False, addend=heads)], stream=stream)
         return res.reshape(x.shape)

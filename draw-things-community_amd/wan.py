@@ -19,8 +19,8 @@ from typing import Dict, Sequence
 
 import numpy as np
 
-from . import (ACT_GELU_TANH, DensePost, QxTensor, dense_multi, dense_post, layernorm_modulate, qk_norm_rope_,
-               sdpa_segments, _torch)
+from . import (ACT_GELU_TANH, DensePost, QxTensor, _side_stream, dense_multi, dense_post, layernorm_modulate,
+               qk_norm_rope_, sdpa_segments, _torch)
 
 DENSE_NAMES = ("x_q", "x_k", "x_v", "x_o", "x_c_q", "c_o", "x_linear1", "x_out_proj")
 ROW_NORM_NAMES = ("x_norm_q", "x_norm_k", "x_c_norm_q")
@@ -51,10 +51,18 @@ class WanAttentionBlock:
             raise ValueError("x does not match the block's token count and width")
         W, Bv, G = self.weight, self.bias, self.norm
         chunks = [ci.reshape(C) + mi.reshape(C) for ci, mi in zip(c, self.modulation)]  # fp32 adds, 6 x [C]
-        out = x.reshape(hw, C).clone()
+        # the copy that the residual epilogues accumulate into is made on a second stream, beside the self-attention's
+        # projections, which read the original
+        main = stream if stream is not None else torch.cuda.current_stream(x.device)
+        side = _side_stream(x.device)
+        x_in = x.reshape(hw, C)
+        out = torch.empty_like(x_in)
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            out.copy_(x_in)
         f16 = dict(dtype=torch.float16, device=x.device)
         # self-attention
-        xn = layernorm_modulate(out, chunks[1], chunks[0], 1e-6, stream=stream)
+        xn = layernorm_modulate(x_in, chunks[1], chunks[0], 1e-6, stream=stream)
         qkv = torch.empty((hw, 3, h, k), **f16)
         qkv2 = qkv.view(hw, 3 * C)
         dense_multi(xn, [W["x_q"], W["x_k"], W["x_v"]], [Bv["x_q"], Bv["x_k"], Bv["x_v"]],
@@ -64,6 +72,7 @@ class WanAttentionBlock:
         qk_norm_rope_(q4, G["x_norm_q"], 1e-6, False, rot=rot, post_scale=quarter, stream=stream)
         qk_norm_rope_(k4, G["x_norm_k"], 1e-6, False, rot=rot, post_scale=quarter, stream=stream)
         att = sdpa_segments([q4], [k4], [v4], 1.0, stream=stream)
+        main.wait_stream(side)
         dense_post(att.view(hw, C), [W["x_o"]], [Bv["x_o"]],
                    [DensePost(gate=chunks[2], residual=out, keep_output=False)], stream=stream)
         # cross-attention
