@@ -21,8 +21,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdthip.so")
 CSRC = os.path.join(_HERE, "csrc")
 
-DT_OK, DT_INVALID, DT_NO_KERNEL, DT_OOM = 0, -1, -2, -3
-_STATUS = {0: "DT_OK", -1: "DT_INVALID", -2: "DT_NO_KERNEL", -3: "DT_OOM"}
+DT_OK, DT_INVALID, DT_NO_KERNEL, DT_OOM, DT_DEVICE_ERROR = 0, -1, -2, -3, -4
+_STATUS = {0: "DT_OK", -1: "DT_INVALID", -2: "DT_NO_KERNEL", -3: "DT_OOM", -4: "DT_DEVICE_ERROR"}
 
 # every symbol include/dt_hip.h declares
 ABI_SYMBOLS = (
@@ -159,6 +159,39 @@ def _stream_ptr(stream=None):
     return ctypes.c_void_p(s.cuda_stream)
 
 
+class _on:
+    """Makes `stream` torch's current stream for the body of an operator, so that the tensors the operator
+    allocates, the copies it makes (`clone`, `contiguous`) and the kernels it launches are all ordered on that one
+    stream, and torch's allocator ties every temporary's reuse to it.  None = leave the current stream alone."""
+
+    def __init__(self, stream):
+        self.ctx = None if stream is None else _torch().cuda.stream(stream)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+
+
+def _stream_scoped(fn):
+    """Runs an operator with its `stream=` argument as torch's current stream (see _on)."""
+    import functools
+    import inspect
+
+    sig = inspect.signature(fn)
+
+    @functools.wraps(fn)
+    def wrapped(*args, **kwargs):
+        stream = sig.bind(*args, **kwargs).arguments.get("stream")
+        with _on(stream):
+            return fn(*args, **kwargs)
+
+    return wrapped
+
+
 def _f16_cuda(t, name):
     torch = _torch()
     if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float16):
@@ -271,12 +304,13 @@ class QxTensor:
     def dequantize(self, stream=None):
         """fp16 [out, in] tensor (K0): what a CPU read of the same key followed by Tensor<Float16>(from:) holds."""
         torch = _torch()
-        if self.qbits == 16:
-            return self.data.clone()
-        out = torch.empty(self.shape, dtype=torch.float16, device=self.data.device)
-        w = self._c()
-        _check("dt_depalettize_f16", lib().dt_depalettize_f16(_stream_ptr(stream), ctypes.byref(w), out.data_ptr()))
-        return out
+        with _on(stream):
+            if self.qbits == 16:
+                return self.data.clone()
+            out = torch.empty(self.shape, dtype=torch.float16, device=self.data.device)
+            w = self._c()
+            _check("dt_depalettize_f16", lib().dt_depalettize_f16(_stream_ptr(stream), ctypes.byref(w), out.data_ptr()))
+            return out
 
 
 # --------------------------------------------------------------------------
@@ -347,14 +381,15 @@ def dense_multi(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object
                 stream=None, epilogues: Optional[Sequence[Optional[HeadEpilogue]]] = None):
     """Several Dense ops that share the input, one launch (x_q / x_k / x_v).  `epilogues[i]` (optional) fuses the
     per-head RMSNorm / RoPE that follows projection i."""
-    x2, M, K, n, W, B, Y, LDY, E, outs = _marshal_dense(x, weights, biases, outs, epilogues)
-    if E is None:
-        st = lib().dt_dense_qx_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, flags)
-        _check("dt_dense_qx_f16", st)
-    else:
-        st = lib().dt_dense_qx_heads_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, E, flags)
-        _check("dt_dense_qx_heads_f16", st)
-    return _shape_outs(x, M, outs)
+    with _on(stream):
+        x2, M, K, n, W, B, Y, LDY, E, outs = _marshal_dense(x, weights, biases, outs, epilogues)
+        if E is None:
+            st = lib().dt_dense_qx_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, flags)
+            _check("dt_dense_qx_f16", st)
+        else:
+            st = lib().dt_dense_qx_heads_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, E, flags)
+            _check("dt_dense_qx_heads_f16", st)
+        return _shape_outs(x, M, outs)
 
 
 ACT_NONE, ACT_GELU_TANH, ACT_SWISH, ACT_GELU_ERF = 0, 1, 2, 3
@@ -384,6 +419,10 @@ def _marshal_posts(posts, weights, M, Y, outs):
             P[i] = _DensePost(ACT_NONE, None, None, 0, 1.0, None, 0, None, None, 0)
             continue
         N = weights[i].shape[0]
+        if float(p.scale) == 0.0:
+            # dt_dense_post.scale == 0 means "no scale" in the C ABI (a zero-initialised struct is a plain Dense)
+            raise ValueError("DensePost.scale must not be 0 (the library reads 0 as 'no scale'); a zero result "
+                             "needs no Dense")
         g16 = g32 = None
         if p.gate is not None:
             if isinstance(p.gate, torch.Tensor) and p.gate.dtype == torch.float32:  # product formed in fp32 (Wan)
@@ -430,10 +469,11 @@ def dense_post(x, weights: Sequence[QxTensor], biases: Sequence[Optional[object]
     """Dense ops sharing `x`, each followed by its DensePost tail inside the GEMM epilogue (the feed-forward's
     linear1 -> GELU and the gated residual additions of a transformer block).  Returns the fp16 outputs (None where
     a projection only accumulates into its residual)."""
-    x2, M, K, n, W, B, Y, LDY, _, outs = _marshal_dense(x, weights, biases, outs, None)
-    P = _marshal_posts(posts, weights, M, Y, outs)
-    st = lib().dt_dense_qx_post_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, P, flags)
-    _check("dt_dense_qx_post_f16", st)
+    with _on(stream):
+        x2, M, K, n, W, B, Y, LDY, _, outs = _marshal_dense(x, weights, biases, outs, None)
+        P = _marshal_posts(posts, weights, M, Y, outs)
+        st = lib().dt_dense_qx_post_f16(_stream_ptr(stream), M, K, x2.data_ptr(), x2.stride(0), W, n, B, Y, LDY, P, flags)
+        _check("dt_dense_qx_post_f16", st)
     lead = tuple(x.shape[:-1])
     return [None if o is None else (o.reshape(lead + (o.shape[-1],)) if o.shape[0] == M and o.is_contiguous() else o)
             for o in outs]
@@ -444,6 +484,11 @@ def dense_grouped(problems: Sequence[dict], flags: int = 0, stream=None):
     problem is a dict with the arguments of dense_multi or dense_post: x, weights, biases, and optionally outs and
     either epilogues or posts.  Returns one list of outputs per problem (None where a projection only accumulates
     into its residual)."""
+    with _on(stream):
+        return _dense_grouped(problems, flags, stream)
+
+
+def _dense_grouped(problems, flags, stream):
     keep = [_marshal_dense(p["x"], p["weights"], p["biases"], p.get("outs"), p.get("epilogues")) for p in problems]
     G = (_DenseGroup * len(keep))()
     cast = lambda a: None if a is None else ctypes.addressof(a)  # the arrays stay alive in `keep` until the call returns
@@ -504,8 +549,14 @@ class LoRADense:
     def _padded(self):
         """The pair with the rank padded by zero rows / columns to the tiled kernel's K granule (64): the zeros add
         nothing, so the results are the same bit for bit, and the up projection avoids the slow any-shape kernel."""
-        key = (self.down.data.data_ptr(), self.up.data.data_ptr())
-        if getattr(self, "_pad_key", None) != key:
+        # keyed on the identity of the pair's tensors (held here, so that their addresses cannot be handed to other
+        # tensors while the cache lives), their in-place modification counters, the rank and the count
+        src = (self.down.data, self.up.data)
+        key = (self.down.data._version, self.up.data._version, self.configuration.rank, self.count,
+               tuple(self.down.shape), tuple(self.up.shape))
+        held = getattr(self, "_pad_src", None)
+        if held is None or held[0] is not src[0] or held[1] is not src[1] or getattr(self, "_pad_key", None) != key:
+            self._pad_src = src
             r = self.configuration.rank
             rp = (r + 63) // 64 * 64
             dn, up = self.down, self.up
@@ -523,7 +574,9 @@ class LoRADense:
         if self.weight is None:
             raise RuntimeError(f"LoRADense {self.name!r}: weight not loaded")
         b = None if self.noBias else self.bias
-        if self.configuration.rank <= 0 or self.down is None or self.up is None:  # no matching LoRA keys: plain Dense
+        # no matching LoRA keys: plain Dense.  A scale of zero makes the branch up(0 * down(x)) = 0 exactly, and
+        # adding zero changes nothing: the same plain Dense
+        if self.configuration.rank <= 0 or self.down is None or self.up is None or self.configuration.scale == 0:
             if post is None:
                 return dense_multi(x, [self.weight], [b], flags=self.flags, stream=stream)[0]
             return dense_post(x, [self.weight], [b], [post], flags=self.flags, stream=stream)[0]
@@ -596,18 +649,20 @@ class RMSNorm:
         self.weight = None
 
     def __call__(self, x, stream=None):
-        y = x.clone()
-        if x.dim() == 4 and self.axis == [3]:
-            return qk_norm_rope_(y, self.weight, self.epsilon, True, stream=stream)
-        if x.dim() == 3 and self.axis == [2]:
-            qk_norm_rope_(_as_heads(y), self.weight, self.epsilon, False, stream=stream)
-            return y
-        raise DtError("RMSNorm", DT_NO_KERNEL)
+        with _on(stream):
+            y = x.clone()
+            if x.dim() == 4 and self.axis == [3]:
+                return qk_norm_rope_(y, self.weight, self.epsilon, True, stream=stream)
+            if x.dim() == 3 and self.axis == [2]:
+                qk_norm_rope_(_as_heads(y), self.weight, self.epsilon, False, stream=stream)
+                return y
+            raise DtError("RMSNorm", DT_NO_KERNEL)
 
 
 MOD_F16, MOD_F32, MOD_AFFINE_F32 = 0, 1, 2
 
 
+@_stream_scoped
 def layernorm_modulate(x, scale=None, shift=None, epsilon: float = 1e-6, out=None, stream=None, affine: bool = False):
     """LayerNorm(epsilon:, axis: [last], elementwiseAffine: false) of the fp32 stream `x` [..., C], then the adaLN
     modulation, fp16 out.  fp16 `scale` / `shift` [C]: `norm(x).to(.Float16) .* scale + shift` (Models/Flux1.swift:
@@ -645,6 +700,7 @@ def layernorm_modulate(x, scale=None, shift=None, epsilon: float = 1e-6, out=Non
     return out.reshape(tuple(x.shape[:-1]) + (C,)) if out.is_contiguous() else out
 
 
+@_stream_scoped
 def layernorm16(x, weight=None, bias=None, epsilon: float = 1e-5, out=None, stream=None):
     """LayerNorm(epsilon:, axis: [last]) with fp16 affine `weight` / `bias` [C] on an fp16 tensor [..., C], fp16 out
     (the norms of a UNet transformer block, Models/UNet.swift:530, 544, 554)."""
@@ -706,9 +762,10 @@ class Functional:
     @staticmethod
     def cmul(left, right, stream=None):
         """Complex multiply on adjacent pairs; `right` is the [1, S, 1, D] (or [S, D]) rotary table."""
-        y = left.clone()
-        rot = right.reshape(-1, right.shape[-1]).contiguous()
-        return qk_norm_rope_(y, None, 0.0, True, rot=rot, stream=stream)
+        with _on(stream):
+            y = left.clone()
+            rot = right.reshape(-1, right.shape[-1]).contiguous()
+            return qk_norm_rope_(y, None, 0.0, True, rot=rot, stream=stream)
 
 
 class ScaledDotProductAttention:
@@ -730,6 +787,7 @@ class ScaledDotProductAttention:
                              stream=stream)
 
 
+@_stream_scoped
 def sdpa_segments(q_segs, k_segs, v_segs, scale, gamma_q=None, gamma_k=None, rot_q=None, rot_k=None,
                   eps: float = 1e-6, Wo=None, bo=None, out=None, stream=None):
     """Attention over a joint sequence given as segments (text || image without a concat).

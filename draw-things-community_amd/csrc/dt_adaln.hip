@@ -258,7 +258,7 @@ DT_EXPORT dt_status dt_layernorm_modulate_f16(dt_stream stream, int64_t M, int64
   const uintptr_t vec_align = mod == DT_MOD_F16 ? 1 : 3;
   if ((reinterpret_cast<uintptr_t>(scale) & vec_align) || (reinterpret_cast<uintptr_t>(shift) & vec_align)) return DT_INVALID;
   if ((M + 3) / 4 > 0x7fffffff) return DT_NO_KERNEL;
-  if (!device_ok()) return DT_NO_KERNEL;
+  if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
   AdaLnArgs a{X, ldx, M, C, scale, shift, eps, Y, ldy};
   const bool vec = (C % 4 == 0) && (ldx % 4 == 0) && (ldy % 4 == 0) && (reinterpret_cast<uintptr_t>(X) & 15) == 0 &&
                    (reinterpret_cast<uintptr_t>(Y) & 7) == 0 &&
@@ -281,7 +281,7 @@ DT_EXPORT dt_status dt_layernorm_f16(dt_stream stream, int64_t M, int64_t C, con
         reinterpret_cast<uintptr_t>(beta)) & 1) != 0)
     return DT_INVALID;
   if ((M + 3) / 4 > 0x7fffffff) return DT_NO_KERNEL;
-  if (!device_ok()) return DT_NO_KERNEL;
+  if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
   const LayerNorm16Args a{X, ldx, M, C, gamma, beta, eps, Y, ldy};
   const bool vec = (C % 8 == 0) && (ldx % 8 == 0) && (ldy % 8 == 0) && C <= 8 * 512 &&
                    ((reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Y) | reinterpret_cast<uintptr_t>(gamma) |

@@ -6,21 +6,33 @@
 
 namespace dt {
 
-bool device_ok() {
-  // 0 = unknown, 1 = gfx950, 2 = other.  Per-process; a process drives one GPU.
-  static std::atomic<int> state{0};
-  int s = state.load(std::memory_order_acquire);
+constexpr int kMaxDevices = 64;
+
+dt_status device_ready() {
+  // per device ordinal: 0 = unknown, 1 = gfx950, 2 = other
+  static std::atomic<int> state[kMaxDevices];
+  // (hipErrorNotReady is the answer of a stream or event query, not a failure)
+  if (const hipError_t pending = hipPeekAtLastError(); pending != hipSuccess && pending != hipErrorNotReady)
+    return DT_DEVICE_ERROR;  // not ours: left for its owner
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();  // this query's own failure
+    return DT_DEVICE_ERROR;
+  }
+  if (dev < 0 || dev >= kMaxDevices) return DT_NO_KERNEL;
+  int s = state[dev].load(std::memory_order_acquire);
   if (s == 0) {
-    int dev = 0;
     hipDeviceProp_t prop;
     s = 2;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) {
+    if (hipGetDeviceProperties(&prop, dev) == hipSuccess) {
       const char* a = prop.gcnArchName;
       if (a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0') s = 1;
+    } else {
+      (void)hipGetLastError();
     }
-    state.store(s, std::memory_order_release);
+    state[dev].store(s, std::memory_order_release);
   }
-  return s == 1;
+  return s == 1 ? DT_OK : DT_NO_KERNEL;
 }
 
 }  // namespace dt
@@ -29,7 +41,7 @@ DT_EXPORT const char* dt_version(void) { return "dthip 0.1 (gfx950)"; }
 
 DT_EXPORT dt_status dt_init(int device) {
   if (hipSetDevice(device) != hipSuccess) return DT_INVALID;
-  return dt::device_ok() ? DT_OK : DT_NO_KERNEL;
+  return dt::device_ready();
 }
 
 DT_EXPORT int64_t dt_qx_bytes(int32_t qbits, int32_t nib, int64_t count) {

@@ -19,16 +19,33 @@ typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
 
 namespace dt {
 
-// True when the current device is a gfx950 part; cached per process.
-bool device_ok();
+// DT_OK when the calling thread's current device is a gfx950 part (cached per device ordinal) and the runtime holds
+// no earlier error; DT_NO_KERNEL for any other architecture; DT_DEVICE_ERROR when an error is already pending on
+// the runtime (a fault of earlier work, the caller's or anyone's: it is left in place for its owner to read, and
+// nothing is enqueued on top of it).
+dt_status device_ready();
 
 inline hipStream_t as_stream(dt_stream s) { return reinterpret_cast<hipStream_t>(s); }
 
-// Launch errors (bad configuration) surface here; execution errors are the
-// stream owner's to observe.
+// Result of the launch just made.  device_ready() has established that no error was pending before it, so what
+// hipGetLastError() returns here belongs to this launch: a configuration the device cannot run (grid, block, LDS or
+// register budget, missing code object) is the library's own "no kernel for this request"; bad arguments are
+// DT_INVALID; anything else (the device was lost, an asynchronous fault surfaced in between) is DT_DEVICE_ERROR.
 inline dt_status launch_status() {
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? DT_OK : DT_INVALID;
+  const hipError_t e = hipGetLastError();
+  switch (e) {
+    case hipSuccess: return DT_OK;
+    case hipErrorInvalidConfiguration:
+    case hipErrorLaunchOutOfResources:
+    case hipErrorInvalidDeviceFunction:
+    case hipErrorNoBinaryForGpu:
+    case hipErrorSharedObjectInitFailed: return DT_NO_KERNEL;
+    case hipErrorInvalidValue:
+    case hipErrorInvalidDevicePointer:
+    case hipErrorInvalidResourceHandle: return DT_INVALID;
+    case hipErrorOutOfMemory: return DT_OOM;
+    default: return DT_DEVICE_ERROR;
+  }
 }
 
 __device__ __forceinline__ half_t bits_to_half(uint16_t b) {

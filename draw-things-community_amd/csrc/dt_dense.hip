@@ -389,7 +389,7 @@ DT_EXPORT dt_status dt_dense_qx_heads_f16(dt_stream stream, int64_t M, int64_t K
   dt_status st = validate_group(h);
   if (st != DT_OK) return st;
   if (M == 0) return DT_OK;
-  if (!device_ok()) return DT_NO_KERNEL;
+  if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
   return run_group(as_stream(stream), h);
 }
 
@@ -403,7 +403,7 @@ DT_EXPORT dt_status dt_dense_qx_post_f16(dt_stream stream, int64_t M, int64_t K,
   dt_status st = validate_group(h);
   if (st != DT_OK) return st;
   if (M == 0) return DT_OK;
-  if (!device_ok()) return DT_NO_KERNEL;
+  if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
   return run_group(as_stream(stream), h);
 }
 
@@ -423,7 +423,7 @@ DT_EXPORT dt_status dt_dense_qx_grouped_f16(dt_stream stream, int32_t n_groups, 
     if (h.M > 0) hs[n++] = h;
   }
   if (n == 0) return DT_OK;
-  if (!device_ok()) return DT_NO_KERNEL;
+  if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
   hipStream_t s = as_stream(stream);
   dt_status st = DT_OK;
   if (run_groups_fused(s, hs, n, &st)) return st;

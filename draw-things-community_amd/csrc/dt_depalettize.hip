@@ -63,7 +63,7 @@ DT_EXPORT dt_status dt_depalettize_f16(dt_stream stream, const dt_qx_weight* w, 
   if (!w->data || !out) return DT_INVALID;
   if (w->qbits < 4 || w->qbits > 8 || w->nib <= 0) return DT_INVALID;
   if ((reinterpret_cast<uintptr_t>(out) & 1) != 0) return DT_INVALID;
-  if (!device_ok()) return DT_NO_KERNEL;
+  if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
   hipStream_t s = as_stream(stream);
   const uint8_t* packed = static_cast<const uint8_t*>(w->data);
   int64_t done = 0;

@@ -287,7 +287,7 @@ DT_EXPORT dt_status dt_qk_norm_rope_f16(dt_stream stream, dt_view4 x, int32_t B,
     return DT_INVALID;
   if (rot && ((reinterpret_cast<uintptr_t>(rot) & 3) || rot_pos0 < 0)) return DT_INVALID;
   if (gamma && !norm_per_head && x.stride_h != D) return DT_INVALID;
-  if (!device_ok()) return DT_NO_KERNEL;
+  if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
   QkPrepArgs a;
   a.src = static_cast<const uint16_t*>(x.ptr);
   a.dst = static_cast<uint16_t*>(x.ptr);

@@ -60,7 +60,7 @@ DT_EXPORT dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t
     if (k_seg[i].len > 0 && (!view_ok(k_seg[i].view, 8) || !view_ok(v_seg[i].view, 8))) return DT_INVALID;
   if (!o.ptr || (reinterpret_cast<uintptr_t>(o.ptr) & 7) || o.stride_b % 4 || o.stride_s % 4) return DT_INVALID;
   if (!Wo && o.stride_h % 4) return DT_INVALID;
-  if (!device_ok()) return DT_NO_KERNEL;
+  if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
 
   const size_t need = dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, prep ? 1 : 0, Wo ? 1 : 0);
   if (need > 0) {

@@ -15,8 +15,10 @@ two of the codecs give the same length for one element count.  Blobs that match 
 length (the reference also compresses small tensors with its `ezm7` coder) and blobs kept in the sidecar are reported
 as unreadable rather than guessed at.
 """
+import os
 import sqlite3
 import struct
+import urllib.parse
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -55,15 +57,26 @@ class TensorInfo:
 class Store:
     """`graph.openStore(path)`: `keys`, `read(key, codec:)`, `write(key, tensor:)` over the container's SQLite file."""
 
-    def __init__(self, path: str, codecs: Optional[Dict[str, Tuple[int, int]]] = None):
-        self.path = path
+    def __init__(self, path: str, codecs: Optional[Dict[str, Tuple[int, int]]] = None, mode: str = "r"):
+        """mode "r" (default): the file must exist and is opened read-only, as the reference's own reader checks
+        first (Scripts/qwen35_gguf_quant_csv.py:113-121); "w": opened read-write, created with an empty `tensors`
+        table if missing."""
+        if mode not in ("r", "w"):
+            raise ValueError("mode must be 'r' or 'w'")
+        self.path, self.mode = path, mode
         self.codecs = dict(CODEC if codecs is None else codecs)
-        self.db = sqlite3.connect(path)
-        self.db.execute("CREATE TABLE IF NOT EXISTS tensors (name TEXT, type INTEGER, format INTEGER, datatype INTEGER, "
-                        "dim BLOB, data BLOB, PRIMARY KEY (name))")
+        if mode == "r":
+            if not os.path.isfile(path):
+                raise FileNotFoundError(path)
+            self.db = sqlite3.connect("file:" + urllib.parse.quote(os.path.abspath(path)) + "?mode=ro", uri=True)
+        else:
+            self.db = sqlite3.connect(path)
+            self.db.execute("CREATE TABLE IF NOT EXISTS tensors (name TEXT, type INTEGER, format INTEGER, datatype INTEGER, "
+                            "dim BLOB, data BLOB, PRIMARY KEY (name))")
 
     def close(self):
-        self.db.commit()
+        if self.mode == "w":
+            self.db.commit()
         self.db.close()
 
     def __enter__(self):
@@ -130,7 +143,9 @@ class Store:
 
     def write(self, key: str, tensor, datatype: Optional[str] = None):
         """Stores a numpy array / torch tensor as plain bytes, or a QxTensor's packed stream as it is (the palette
-        fitting of the reference's quantizer is not part of this library)."""
+        fitting of the reference's quantizer is not part of this library).  Needs a store opened with mode "w"."""
+        if self.mode != "w":
+            raise PermissionError(f"{self.path} was opened read-only")
         if isinstance(tensor, QxTensor):
             if tensor.qbits == 16:
                 return self.write(key, tensor.data.cpu().numpy())

@@ -7,7 +7,7 @@
  * DEVICE pointer borrowed for the duration of the enqueue (the call returns
  * once the work is queued on `stream`; it never synchronises the stream).
  * All entry points are re-entrant and stream-ordered; the library keeps no
- * mutable global state apart from a once-per-process device query.
+ * mutable global state apart from a once-per-device architecture query.
  *
  * Status codes mirror the values a ccv_nnc backend `exec` returns, so a shim
  * can map DT_NO_KERNEL to "fall through to the next backend":
@@ -15,6 +15,9 @@
  *   -1  DT_INVALID     bad shape / alignment / NULL pointer / unknown qbits
  *   -2  DT_NO_KERNEL   valid request this library has no kernel for
  *   -3  DT_OOM         workspace too small
+ *   -4  DT_DEVICE_ERROR the HIP runtime already held an error when the call was made (left in place for its owner;
+ *                      nothing was enqueued), or the device failed under the launch; no ccv counterpart: a shim
+ *                      maps it to CCV_NNC_EXEC_INVALID
  *
  * The operator surface this replaces is the one the reference's model
  * builders call (reference paths relative to Libraries/SwiftDiffusion/Sources):
@@ -40,6 +43,7 @@ typedef int32_t dt_status;
 #define DT_INVALID (-1)
 #define DT_NO_KERNEL (-2)
 #define DT_OOM (-3)
+#define DT_DEVICE_ERROR (-4)
 
 /* A hipStream_t passed as an opaque pointer; NULL is the default stream. */
 typedef void* dt_stream;
@@ -85,8 +89,8 @@ typedef struct {
 /* Library identification; never NULL. */
 const char* dt_version(void);
 
-/* Checks that `device` is a gfx950 part and warms the per-process device
- * query.  Optional: every entry point does the same check lazily.
+/* Makes `device` the calling thread's current device, checks that it is a gfx950 part and warms the per-device
+ * query.  Optional: every entry point does the same check lazily for whichever device is current.
  * Returns DT_NO_KERNEL on any other architecture. */
 dt_status dt_init(int device);
 

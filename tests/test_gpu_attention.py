@@ -427,3 +427,83 @@ def test_block_step_replays_as_hip_graph(dthip, oracle, torch_cuda):
             assert torch.equal(a_, b_)
         step()
         torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("B,S,H,D", [(1, 1024, 2, 128), (2, 512, 8, 40), (1, 1536, 3, 128)])
+def test_sdpa_vs_op_by_op_fp16_graph(dthip, oracle, torch_cuda, B, S, H, D):
+    """The `.none` attention path of the reference (Matmul(transposeB:) -> softmax -> Matmul on fp16 tensors with the
+    scale applied to Q first, Models/Flux1.swift:192-223, Models/UNet.swift:217-262) is what an op-by-op CPU run
+    executes: scaled Q, scores and probabilities are each stored as fp16 between the three ops.  The fused kernel
+    keeps them in fp32; the two must agree within the attention bar (max-abs 2e-2, rel-RMS 1e-3)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(S + D)
+    q, k, v = rand_qkv(rng, B, S, S, H, H, D)
+    scale = 1 / np.sqrt(D)
+    print("sdpa vs op-by-op graph", B, S, H, D, flush=True)
+    got = dthip.ScaledDotProductAttention(scale=scale, flags=dthip.GEMMFlag.Float16)(
+        to_dev(torch, q), to_dev(torch, k), to_dev(torch, v)).cpu().numpy()
+    want = oracle.C.sdpa(q, k, v, scale, round_mid=1)
+    mx, rr = oracle.err_stats(got, want)
+    print("  gap to the op-by-op fp16 graph: max-abs %.3e rel-RMS %.3e" % (mx, rr), flush=True)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+def test_sdpa_sd15_full_size_sampled(dthip, oracle, torch_cuda):
+    """SD 1.5 UNet attention at its full shape (batch 2, 8 heads x 40, 64 x 64 latent = 4096 tokens): self-attention
+    over 4096 keys and cross-attention over 77 keys with the unify-heads projection fused
+    (Models/UNet.swift:122-155, 311-319).  Sampled rows against the oracle, constant-V over the whole output."""
+    torch = torch_cuda
+    rng = np.random.default_rng(40)
+    B, S, T, H, D = 2, 4096, 77, 8, 40
+    scale = 1 / np.sqrt(D)
+    q, k, v = rand_qkv(rng, B, S, S, H, H, D)
+    qd, kd, vd = (to_dev(torch, t) for t in (q, k, v))
+    print("sdpa sd15 self full size", flush=True)
+    got = dthip.ScaledDotProductAttention(scale=scale)(qd, kd, vd).cpu().numpy()
+    rows = np.sort(rng.choice(S, size=40, replace=False))
+    rows[0], rows[-1] = 0, S - 1
+    want = oracle.C.sdpa(np.ascontiguousarray(q[:, rows]), k, v, scale)
+    mx, rr = oracle.err_stats(got[:, rows], want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+    vc = torch.from_numpy(f16(rng.standard_normal((1, 1, H, D)))).cuda().expand(B, S, H, D).contiguous()
+    oc = dthip.ScaledDotProductAttention(scale=scale)(qd, kd, vc)
+    assert float((oc.float() - vc.float()).abs().max()) <= 2e-3
+    # cross-attention, 77 keys, fused output projection
+    kc, vcx = f16(rng.standard_normal((B, T, H, D))), f16(rng.standard_normal((B, T, H, D)))
+    Wo = f16(rng.standard_normal((H * D, H * D)) * 0.05)
+    bo = f16(rng.standard_normal(H * D) * 0.05)
+    op = dthip.ScaledDotProductAttention(scale=scale, multiHeadOutputProjectionFused=True)
+    op.weight, op.bias = to_dev(torch, Wo), to_dev(torch, bo)
+    print("sdpa sd15 cross full size, fused unify-heads", flush=True)
+    gotc = op(qd, to_dev(torch, kc), to_dev(torch, vcx)).cpu().numpy()
+    assert gotc.shape == (B, S, H * D)
+    att = oracle.C.sdpa(np.ascontiguousarray(q[:, rows]), kc, vcx, scale).reshape(B * rows.size, H * D)
+    wantc = oracle.C.dense(att, Wo, bo).reshape(B, rows.size, H * D)
+    mx, rr = oracle.err_stats(gotc[:, rows], wantc)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+def test_sdpa_wan_cross_attention_full_size_sampled(dthip, oracle, torch_cuda):
+    """Wan cross-attention at its full shape: 32760 query tokens against 512 text keys, 40 heads x 128, scale
+    1/sqrt(128) (Models/Wan.swift:163-174).  Sampled rows of two heads against the oracle; constant-V property."""
+    torch = torch_cuda
+    rng = np.random.default_rng(41)
+    B, Sq, Skv, H, D = 1, 32760, 512, 40, 128
+    gen = torch.Generator(device="cuda").manual_seed(41)
+    qd = torch.randn((B, Sq, H, D), device="cuda", generator=gen).half()
+    kd = torch.randn((B, Skv, H, D), device="cuda", generator=gen).half()
+    vd = torch.randn((B, Skv, H, D), device="cuda", generator=gen).half()
+    scale = 1 / np.sqrt(D)
+    print("sdpa wan cross full size", flush=True)
+    got = dthip.ScaledDotProductAttention(scale=scale)(qd, kd, vd)
+    rows = np.sort(rng.choice(Sq, size=64, replace=False))
+    rows[0], rows[-1] = 0, Sq - 1
+    rt = torch.from_numpy(rows).cuda()
+    for h in (0, 17, 39):
+        want = oracle.C.sdpa(np.ascontiguousarray(qd[:, rt, h:h + 1].cpu().numpy()), np.ascontiguousarray(kd[:, :, h:h + 1].cpu().numpy()),
+                             np.ascontiguousarray(vd[:, :, h:h + 1].cpu().numpy()), scale)
+        mx, rr = oracle.err_stats(got[:, rt, h:h + 1].cpu().numpy(), want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (h, mx, rr)
+    vc = torch.randn((1, 1, H, D), device="cuda", generator=gen).half().expand(B, Skv, H, D).contiguous()
+    oc = dthip.ScaledDotProductAttention(scale=scale)(qd, kd, vc)
+    assert float((oc.float() - vc[:, :1].float()).abs().max()) <= 2e-3

@@ -658,3 +658,105 @@ def test_dense_post_activations_over_every_fp16_input(dthip, oracle, torch_cuda)
         assert np.array_equal(np.isfinite(got), np.isfinite(want)), act
         ok = np.isfinite(want)
         assert int(ulps(got, want)[ok].max()) <= 1, (act, int(ulps(got, want)[ok].max()))
+
+
+def test_dense_q8p_full_size_sampled(dthip, oracle, torch_cuda):
+    """"Palettized Dense alone" at its full shape with 8-bit indices: M 4608, K 3072, three N 3072 q8p weights (256-entry
+    palettes, 16384 elements per block: a block spans 5 1/3 weight rows, so a 256-row tile holds about 50 palettes) in
+    one launch, and the single 3072 -> 3072 output projection.  Sampled rows against the oracle, and the weights the
+    kernel multiplies by checked bit for bit at K = 3072 (X = I makes Y = W^T exactly)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(28)
+    M, K, N, q, nib = 4608, 3072, 3072, 8, 16384
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    ws, packs, biases = [], [], []
+    for i in range(3):
+        w, p = make_weight(dthip, oracle, rng, N, K, q, nib)
+        ws.append(w)
+        packs.append(p)
+        biases.append((rng.standard_normal(N) * 0.02).astype(np.float16))
+    xd = to_dev(torch, X)
+    print("dense q8p full size", flush=True)
+    outs = dthip.dense_multi(xd, ws, [to_dev(torch, b) for b in biases])
+    rows = np.sort(rng.choice(M, size=24, replace=False))
+    rows[0], rows[-1] = 0, M - 1
+    for i in range(3):
+        got = outs[i].cpu().numpy()[rows]
+        want = oracle.C.dense_qx(np.ascontiguousarray(X[rows]), packs[i], q, nib, N, biases[i])
+        mx, rr = oracle.err_stats(got, want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (i, mx, rr)
+    one = dthip.dense_multi(xd, [ws[1]], [to_dev(torch, biases[1])])[0]
+    assert torch.equal(one, outs[1])
+    print("dense q8p effective weights at K = 3072", flush=True)
+    eye = torch.eye(K, dtype=torch.float16, device="cuda")
+    for i in (0, 2):
+        Y = dthip.dense_multi(eye, [ws[i]], [None])[0].cpu().numpy()
+        W = oracle.C.depalettize(q, nib, N * K, packs[i]).reshape(N, K)
+        assert np.array_equal(Y.view(np.uint16), np.ascontiguousarray(W.T).view(np.uint16))
+
+
+def test_lora_dense_swap_and_zero_scale(dthip, oracle, torch_cuda):
+    """A second LoRA of the same shape replaces the first (its tensors may land at the addresses the first pair's
+    had: the padded copies must follow the new pair, and an in-place update of a pair too); a scale of zero switches
+    the branch off as `0 * down(x)` does (Models/LoRA.swift:129-134)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(77)
+    M, N, K, q, nib, rank = 200, 256, 192, 6, 4096, 16
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    w, p = make_weight(dthip, oracle, rng, N, K, q, nib, std=0.05)
+    xd = to_dev(torch, X)
+    layer = dthip.LoRADense(N, dthip.LoRANetworkConfiguration(rank, 1.0), noBias=True)
+    layer.weight = w
+    base = oracle.C.dense_qx(X, p, q, nib, N, None)
+    print("lora swap", flush=True)
+    for trial in range(3):
+        down = (rng.standard_normal((rank, K)) * 0.1).astype(np.float16)
+        up = (rng.standard_normal((N, rank)) * 0.1).astype(np.float16)
+        layer.down = layer.up = None          # the old pair is released before the new one is made
+        torch.cuda.empty_cache() if trial == 2 else None
+        layer.down, layer.up = dthip.QxTensor.from_f16(down), dthip.QxTensor.from_f16(up)
+        out = layer(xd).cpu().numpy()
+        want = oracle.np_add16(base, oracle.np_lora_branch16(X, down, up, 1.0))
+        mx, rr = oracle.err_stats(out, want)
+        assert mx <= MAX_ABS and rr <= 2 * REL_RMS, (trial, mx, rr)
+    # in-place update of the current pair
+    down2 = (rng.standard_normal((rank, K)) * 0.1).astype(np.float16)
+    layer.down.data.copy_(to_dev(torch, down2))
+    out = layer(xd).cpu().numpy()
+    want = oracle.np_add16(base, oracle.np_lora_branch16(X, down2, up, 1.0))
+    mx, rr = oracle.err_stats(out, want)
+    assert mx <= MAX_ABS and rr <= 2 * REL_RMS, (mx, rr)
+    # scale 0: the plain Dense
+    zero = dthip.LoRADense(N, dthip.LoRANetworkConfiguration(rank, 0.0), noBias=True)
+    zero.weight, zero.down, zero.up = w, layer.down, layer.up
+    assert torch.equal(zero(xd), dthip.dense_multi(xd, [w], [None])[0])
+    with pytest.raises(ValueError):
+        dthip.dense_post(xd, [w], [None], [dthip.DensePost(scale=0.0)])
+
+
+def test_operators_on_a_side_stream(dthip, oracle, torch_cuda):
+    """`stream=` other than the current stream: the operator's own allocations, copies and launches all go to that
+    stream (clone-then-launch operators such as RMSNorm and cmul, and attention with its workspace)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(78)
+    B, S, H, D = 1, 300, 4, 128
+    x = rng.standard_normal((B, S, H, D)).astype(np.float16)
+    g = (1 + 0.02 * rng.standard_normal(D)).astype(np.float16)
+    rot = dthip.Flux1RotaryPositionEmbedding(15, 20, 0, channels=D).astype(np.float16)
+    side = torch.cuda.Stream()
+    xd, gd, rd = to_dev(torch, x), to_dev(torch, g), to_dev(torch, rot)
+    torch.cuda.synchronize()
+    print("operators on a side stream", flush=True)
+    n = dthip.RMSNorm(epsilon=1e-6, axis=[3])
+    n.weight = gd
+    y = n(xd, stream=side)
+    want_y = oracle.C.rmsnorm(x[0], g, 1e-6)
+    z = dthip.Functional.cmul(to_dev(torch, want_y[None]), rd.reshape(1, S, 1, D), stream=side)
+    o = dthip.sdpa_segments([xd], [xd], [xd], 1 / np.sqrt(D), gamma_q=[gd], gamma_k=[gd], rot_q=rd, rot_k=rd, stream=side)
+    side.synchronize()
+    want_z = oracle.C.cmul(want_y, rot)
+    assert np.all(np.abs(y.cpu().numpy()[0].astype(np.float32) - want_y.astype(np.float32)) <= np.abs(want_y.astype(np.float32)) * 2.0 ** -10 + 2.0 ** -24)
+    assert np.array_equal(z.cpu().numpy()[0].view(np.uint16), want_z.view(np.uint16))
+    want_o = oracle.C.sdpa(want_z[None], want_z[None], x, 1 / np.sqrt(D))
+    mx, rr = oracle.err_stats(o.cpu().numpy(), want_o)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)

@@ -17,7 +17,7 @@ def test_store_to_dense(tmp_path, dthip, oracle):
     packed, _, _ = oracle.synth_qx_weight(rng, N, K, q, nib, 0.05)
     bias = (rng.standard_normal(N) * 0.1).astype(np.float16)
     path = str(tmp_path / "m.ckpt")
-    with store_mod.Store(path) as st:
+    with store_mod.Store(path, mode="w") as st:
         st.write("__dit__[t-x_q-0-0]", dthip.QxTensor.from_packed(packed, q, nib, (N, K), device="cpu"))
         st.write("__dit__[t-x_q-0-1]", bias)
     print("store -> dense", flush=True)

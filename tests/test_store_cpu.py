@@ -3,6 +3,7 @@ codes, the little-endian int32 `dim` array and the key scheme are the ones the r
 (Scripts/qwen35_gguf_quant_csv.py:48-55, 113-135); palettized blobs come from the oracle's packer.  What a real file
 would pin beyond that (how a row marks its codec, compressed blobs, the sidecar) is not covered: parity unpinned."""
 import importlib
+import os
 import sqlite3
 import struct
 
@@ -84,7 +85,10 @@ def test_store_write_round_trip(tmp_path, store_mod, dthip, oracle):
     w = dthip.QxTensor.from_packed(packed, 4, 512, (8, 64), device="cpu")
     f32 = rng.standard_normal((3, 5)).astype(np.float32)
     path = str(tmp_path / "out.ckpt")
-    with store_mod.Store(path) as st:
+    with pytest.raises(FileNotFoundError):   # a reader never creates the file it was asked to read
+        store_mod.Store(path)
+    assert not os.path.exists(path)
+    with store_mod.Store(path, mode="w") as st:
         st.write("a", w)
         st.write("b", f32)
     with store_mod.Store(path) as st:
@@ -92,6 +96,8 @@ def test_store_write_round_trip(tmp_path, store_mod, dthip, oracle):
         assert (back.qbits, back.nib, back.shape) == (4, 512, (8, 64))
         assert np.array_equal(back.data.numpy()[: packed.size], packed)
         assert np.array_equal(st.read("b", (), device="cpu").numpy(), f32)
+        with pytest.raises(PermissionError):   # opened read-only
+            st.write("c", f32)
     # the file is what the reference's own script expects: name, datatype, dim columns of table `tensors`
     rows = sqlite3.connect(path).execute("select name, datatype, dim from tensors order by name").fetchall()
     assert [r[0] for r in rows] == ["a", "b"] and rows[0][1] == 131072 and rows[1][1] == 16384
