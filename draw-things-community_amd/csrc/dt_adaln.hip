@@ -13,7 +13,7 @@ __device__ __forceinline__ float wave_sum64(float v) {
   return v;
 }
 
-__device__ __forceinline__ float round16(float v) { return (float)(half_t)v; }
+__device__ __forceinline__ float round16(float v) { return round_f16(v); }
 
 // One normalised value through the modulation (sc, sh already widened to float).
 //   DT_MOD_F16: fp16(fp16(fp16(n) * scale) + shift), scale and shift fp16

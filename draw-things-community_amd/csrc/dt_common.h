@@ -34,7 +34,8 @@ inline hipStream_t as_stream(dt_stream s) { return reinterpret_cast<hipStream_t>
 inline dt_status launch_status() {
   const hipError_t e = hipGetLastError();
   switch (e) {
-    case hipSuccess: return DT_OK;
+    case hipSuccess:
+    case hipErrorNotReady: return DT_OK;  // (the answer of someone's stream or event query, not a failure)
     case hipErrorInvalidConfiguration:
     case hipErrorLaunchOutOfResources:
     case hipErrorInvalidDeviceFunction:
@@ -56,6 +57,15 @@ __device__ __forceinline__ uint16_t half_to_bits(half_t h) {
 }
 
 #if defined(__HIPCC__)
+// fp32 -> fp16 -> fp32 as a rounding step of its own.  The empty asm keeps the compiler from folding the arithmetic
+// that produced `v` and the conversion into one mixed-precision instruction (v_fma_mixlo_f16 rounds the exact
+// product-sum to fp16 once; the op-by-op graph rounds it to fp32 first and to fp16 second, and the two differ by an
+// ulp in about one result in 2^15).
+__device__ __forceinline__ float round_f16(float v) {
+  asm volatile("" : "+v"(v));
+  return (float)(half_t)v;
+}
+
 // Combine the two half-waves (lanes l and l ^ 32 hold the same matrix column) without touching LDS:
 // v_permlane32_swap of a register with a copy of itself leaves {low, low} and {high, high}.
 __device__ __forceinline__ void halves32(float v, float& lo, float& hi) {

@@ -45,7 +45,7 @@ __global__ void __launch_bounds__(256) dense_qx_generic_kernel(const uint16_t* _
     }
   }
   if (bias) acc += (float)bits_to_half(bias[ni]);
-  float v = (float)(half_t)acc;
+  float v = round_f16(acc);
   v = post_value(v, scale, add != nullptr, add ? (float)bits_to_half(add[mi * ld_add + ni]) : 0.f, mul != nullptr,
                  mul ? (float)bits_to_half(mul[mi * ld_mul + ni]) : 1.f, act, gate != nullptr,
                  gate ? (float)bits_to_half(gate[ni]) : 1.0f);

@@ -64,13 +64,13 @@ __device__ __forceinline__ float act_swish(float x) {
 __device__ __forceinline__ float act_gelu_erf(float x) { return 0.5f * x * erfcf(x * -0.7071067811865476f); }
 __device__ __forceinline__ float post_value(float v, float scale, bool has_add, float add, bool has_mul, float mul, int act,
                                             bool has_gate, float gate) {
-  if (scale != 1.0f) v = (float)(half_t)(v * scale);
-  if (has_add) v = (float)(half_t)(v + add);
-  if (has_mul) v = (float)(half_t)(v * mul);
+  if (scale != 1.0f) v = round_f16(v * scale);
+  if (has_add) v = round_f16(v + add);
+  if (has_mul) v = round_f16(v * mul);
   if (act == DT_ACT_GELU_TANH) v = (float)(half_t)act_gelu_tanh(v);
   else if (act == DT_ACT_SWISH) v = (float)(half_t)act_swish(v);
   else if (act == DT_ACT_GELU_ERF) v = (float)(half_t)act_gelu_erf(v);
-  if (has_gate) v = (float)(half_t)(v * gate);
+  if (has_gate) v = round_f16(v * gate);
   return v;
 }
 
@@ -750,7 +750,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
           ss = row16_sum(ss);
           const float inv = 1.0f / sqrtf(ss / (float)WN + w.eps);
 #pragma unroll
-          for (int e = 0; e < 8; e++) v[e] = (float)(half_t)(v[e] * inv * gt[e]);
+          for (int e = 0; e < 8; e++) v[e] = round_f16(v[e] * inv * gt[e]);
         }
         if (w.rot) {
           uint4_t rr;
@@ -765,8 +765,8 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
           for (int q = 0; q < 4; q++) {
             const float cs = lo16(rr[q]), sn = hi16(rr[q]);
             const float re = v[2 * q], im = v[2 * q + 1];
-            v[2 * q] = (float)(half_t)(re * cs - im * sn);
-            v[2 * q + 1] = (float)(half_t)(re * sn + im * cs);
+            v[2 * q] = round_f16(re * cs - im * sn);
+            v[2 * q + 1] = round_f16(re * sn + im * cs);
           }
         }
       }
@@ -814,7 +814,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         }
         // post_value's steps, each over the row's 8 values under one uniform test (a step that is off costs a
         // branch, not eight selects)
-        const auto rh = [](float x) { return (float)(half_t)x; };
+        const auto rh = [](float x) { return round_f16(x); };
         if (w.scale != 1.0f) {
 #pragma unroll
           for (int e = 0; e < 8; e++) v[e] = rh(v[e] * w.scale);

@@ -12,7 +12,7 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-__device__ __forceinline__ float round_h(float v) { return (float)(half_t)v; }
+__device__ __forceinline__ float round_h(float v) { return round_f16(v); }
 
 // normalise-rotate-scale one (re, im) pair that is already in registers
 __device__ __forceinline__ uint32_t finish_pair(float a, float b, float inv, const uint16_t* gamma, int p,

@@ -744,14 +744,14 @@ def test_operators_on_a_side_stream(dthip, oracle, torch_cuda):
     g = (1 + 0.02 * rng.standard_normal(D)).astype(np.float16)
     rot = dthip.Flux1RotaryPositionEmbedding(15, 20, 0, channels=D).astype(np.float16)
     side = torch.cuda.Stream()
-    xd, gd, rd = to_dev(torch, x), to_dev(torch, g), to_dev(torch, rot)
-    torch.cuda.synchronize()
+    want_y = oracle.C.rmsnorm(x[0], g, 1e-6)
+    xd, gd, rd, yd = to_dev(torch, x), to_dev(torch, g), to_dev(torch, rot), to_dev(torch, want_y[None])
+    torch.cuda.synchronize()  # the uploads above ran on the default stream
     print("operators on a side stream", flush=True)
     n = dthip.RMSNorm(epsilon=1e-6, axis=[3])
     n.weight = gd
     y = n(xd, stream=side)
-    want_y = oracle.C.rmsnorm(x[0], g, 1e-6)
-    z = dthip.Functional.cmul(to_dev(torch, want_y[None]), rd.reshape(1, S, 1, D), stream=side)
+    z = dthip.Functional.cmul(yd, rd.reshape(1, S, 1, D), stream=side)
     o = dthip.sdpa_segments([xd], [xd], [xd], 1 / np.sqrt(D), gamma_q=[gd], gamma_k=[gd], rot_q=rd, rot_k=rd, stream=side)
     side.synchronize()
     want_z = oracle.C.cmul(want_y, rot)
