@@ -39,7 +39,10 @@ ABI_SYMBOLS = (
     "dt_layernorm_f16",
     "dt_sdpa_f16",
     "dt_sdpa_workspace_bytes",
+    "dt_sdpa_f16_static",
 )
+
+STATIC_SCRATCH_BYTES = 64 << 20  # DT_SDPA_STATIC_SCRATCH_BYTES
 
 
 class DtError(RuntimeError):
@@ -136,6 +139,8 @@ def lib():
         L.dt_sdpa_f16.argtypes = [vp, i32, i32, i32, i32, i32, ctypes.POINTER(_Segment), i32,
                                   ctypes.POINTER(_Segment), ctypes.POINTER(_Segment), vp, vp, f32, _View4, f32,
                                   vp, vp, vp, ctypes.c_size_t]
+        L.dt_sdpa_f16_static.restype = i32
+        L.dt_sdpa_f16_static.argtypes = L.dt_sdpa_f16.argtypes[:-2]
         L.dt_sdpa_workspace_bytes.restype = ctypes.c_size_t
         L.dt_sdpa_workspace_bytes.argtypes = [i32, i32, i32, i32, i64, i64, i32, i32]
         _lib = L
@@ -789,9 +794,12 @@ class ScaledDotProductAttention:
 
 @_stream_scoped
 def sdpa_segments(q_segs, k_segs, v_segs, scale, gamma_q=None, gamma_k=None, rot_q=None, rot_k=None,
-                  eps: float = 1e-6, Wo=None, bo=None, out=None, stream=None):
+                  eps: float = 1e-6, Wo=None, bo=None, out=None, stream=None, static_scratch: bool = False):
     """Attention over a joint sequence given as segments (text || image without a concat).
-    gamma_q / gamma_k: per-segment per-head RMSNorm weights (or None); rot_*: [S, D] tables."""
+    gamma_q / gamma_k: per-segment per-head RMSNorm weights (or None); rot_*: [S, D] tables.
+    static_scratch: stage through the library's fixed per-GPU array (dt_sdpa_f16_static) instead of a workspace
+    allocated here; with `out` given the call then allocates nothing.  Requests beyond STATIC_SCRATCH_BYTES raise
+    DtError(DT_OOM); calls that may overlap on one GPU must not both use it."""
     torch = _torch()
     L = lib()
     for t in list(q_segs) + list(k_segs) + list(v_segs):
@@ -820,17 +828,21 @@ def sdpa_segments(q_segs, k_segs, v_segs, scale, gamma_q=None, gamma_k=None, rot
         ov = _View4(out.data_ptr(), out.stride(0), out.stride(1), 0)
     else:
         ov = _view4(out)
+    rq = None if rot_q is None else _f16_cuda(rot_q, "rot_q").data_ptr()
+    rk = None if rot_k is None else _f16_cuda(rot_k, "rot_k").data_ptr()
+    wo = None if Wo is None else _f16_cuda(Wo, "Wo").data_ptr()
+    bo_p = None if bo is None else _f16_cuda(bo, "bo").data_ptr()
+    if static_scratch:
+        st = L.dt_sdpa_f16_static(_stream_ptr(stream), B, Hq, Hk, D, nq, qa, nk, ka, va, rq, rk, eps, ov, scale, wo, bo_p)
+        _check("dt_sdpa_f16_static", st)
+        return out
     need = L.dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, int(prep), int(fused))
     ws = torch.empty(max(need, 256) + 256, dtype=torch.uint8, device=out.device) if need else None
     ws_ptr = None
     if ws is not None:
         ws_ptr = (ws.data_ptr() + 255) & ~255
     st = L.dt_sdpa_f16(
-        _stream_ptr(stream), B, Hq, Hk, D, nq, qa, nk, ka, va,
-        None if rot_q is None else _f16_cuda(rot_q, "rot_q").data_ptr(),
-        None if rot_k is None else _f16_cuda(rot_k, "rot_k").data_ptr(),
-        eps, ov, scale, None if Wo is None else _f16_cuda(Wo, "Wo").data_ptr(),
-        None if bo is None else _f16_cuda(bo, "bo").data_ptr(), ws_ptr, need)
+        _stream_ptr(stream), B, Hq, Hk, D, nq, qa, nk, ka, va, rq, rk, eps, ov, scale, wo, bo_p, ws_ptr, need)
     _check("dt_sdpa_f16", st)
     return out
 

@@ -3,6 +3,7 @@
 
 #include "dt_common.h"
 #include "dt_layout.h"
+#include "dt_sdpa.h"
 
 namespace dt {
 
@@ -41,7 +42,10 @@ DT_EXPORT const char* dt_version(void) { return "dthip 0.1 (gfx950)"; }
 
 DT_EXPORT dt_status dt_init(int device) {
   if (hipSetDevice(device) != hipSuccess) return DT_INVALID;
-  return dt::device_ready();
+  const dt_status st = dt::device_ready();
+  // the device address of this GPU's static scratch (dt_sdpa_f16_static), looked up while `device` is current
+  if (st == DT_OK && !dt::sdpa_static_scratch()) return DT_DEVICE_ERROR;
+  return st;
 }
 
 DT_EXPORT int64_t dt_qx_bytes(int32_t qbits, int32_t nib, int64_t count) {

@@ -25,4 +25,8 @@ struct SdpaArgs {
 
 dt_status sdpa_launch(hipStream_t s, const SdpaArgs& a);
 
+// Device address of the current device's static scratch array (the one dt_sdpa_f16_static uses); looked up once
+// per device.  nullptr on failure.
+void* sdpa_static_scratch();
+
 }  // namespace dt

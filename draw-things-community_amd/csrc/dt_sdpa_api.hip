@@ -1,5 +1,7 @@
 // Host side of the attention entry point: validation, segment tables, the
 // optional norm/rotate staging pass and the optional fused output projection.
+#include <atomic>
+
 #include "dt_common.h"
 #include "dt_qkprep.h"
 #include "dt_sdpa.h"
@@ -30,12 +32,15 @@ DT_EXPORT size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int3
   return bytes;
 }
 
-DT_EXPORT dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D, int32_t n_qseg,
-                                const dt_seq_segment* q_seg, int32_t n_kvseg, const dt_seq_segment* k_seg,
-                                const dt_seq_segment* v_seg, const uint16_t* rot_q, const uint16_t* rot_k, float eps,
-                                dt_view4 o, float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
-                                size_t workspace_bytes) {
-  using namespace dt;
+namespace dt {
+
+// Validation and enqueue shared by dt_sdpa_f16 (caller's workspace) and dt_sdpa_f16_static (the library's own
+// per-device array).  Calls nothing that allocates.
+static dt_status sdpa_enqueue(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D, int32_t n_qseg,
+                              const dt_seq_segment* q_seg, int32_t n_kvseg, const dt_seq_segment* k_seg,
+                              const dt_seq_segment* v_seg, const uint16_t* rot_q, const uint16_t* rot_k, float eps,
+                              dt_view4 o, float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
+                              size_t workspace_bytes) {
   if (B < 0 || Hq <= 0 || Hk <= 0 || D <= 0 || Hq % Hk != 0) return DT_INVALID;
   if (n_qseg <= 0 || n_kvseg <= 0 || !q_seg || !k_seg || !v_seg) return DT_INVALID;
   if (n_qseg > kMaxSeg || n_kvseg > kMaxSeg) return DT_NO_KERNEL;
@@ -203,4 +208,71 @@ DT_EXPORT dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t
   a.o_ss = o.stride_s;
   a.o_sh = o.stride_h;
   return sdpa_launch(s, a);
+}
+
+// ---- the library's own scratch, for callers that cannot allocate ------------------------------------------------
+// One array per GPU (every device that loads this code object holds its own copy at its own address, until the
+// process ends).  In host code the array's name is only a handle for hipGetSymbolAddress; the device address it
+// yields -- looked up once per device, with that device current -- is what kernels and the host side use.
+static __device__ __align__(256) unsigned char scratch[DT_SDPA_STATIC_SCRATCH_BYTES];
+
+static std::atomic<void*> g_scratch_ptr[64];
+
+// Device address of the calling thread's current device's array (nullptr on failure).
+void* sdpa_static_scratch() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* q = nullptr;
+    if (hipGetSymbolAddress(&q, HIP_SYMBOL(scratch)) != hipSuccess || !q) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    g_scratch_ptr[dev].store(q, std::memory_order_release);
+    p = q;
+  }
+  return p;
+}
+
+}  // namespace dt
+
+DT_EXPORT dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D, int32_t n_qseg,
+                                const dt_seq_segment* q_seg, int32_t n_kvseg, const dt_seq_segment* k_seg,
+                                const dt_seq_segment* v_seg, const uint16_t* rot_q, const uint16_t* rot_k, float eps,
+                                dt_view4 o, float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
+                                size_t workspace_bytes) {
+  return dt::sdpa_enqueue(stream, B, Hq, Hk, D, n_qseg, q_seg, n_kvseg, k_seg, v_seg, rot_q, rot_k, eps, o, scale, Wo,
+                          bo, workspace, workspace_bytes);
+}
+
+DT_EXPORT dt_status dt_sdpa_f16_static(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D, int32_t n_qseg,
+                                       const dt_seq_segment* q_seg, int32_t n_kvseg, const dt_seq_segment* k_seg,
+                                       const dt_seq_segment* v_seg, const uint16_t* rot_q, const uint16_t* rot_k,
+                                       float eps, dt_view4 o, float scale, const uint16_t* Wo, const uint16_t* bo) {
+  using namespace dt;
+  if (B < 0 || Hq <= 0 || Hk <= 0 || D <= 0 || n_qseg <= 0 || n_kvseg <= 0 || !q_seg || !k_seg) return DT_INVALID;
+  // the scratch this request needs, by the same rule as dt_sdpa_workspace_bytes
+  int64_t Sq = 0, Skv = 0;
+  bool prep = rot_q || rot_k;
+  for (int i = 0; i < n_qseg; i++) {
+    if (q_seg[i].len < 0) return DT_INVALID;
+    Sq += q_seg[i].len;
+    prep = prep || q_seg[i].gamma;
+  }
+  for (int i = 0; i < n_kvseg; i++) {
+    if (k_seg[i].len < 0) return DT_INVALID;
+    Skv += k_seg[i].len;
+    prep = prep || k_seg[i].gamma;
+  }
+  const size_t need = dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, prep ? 1 : 0, Wo ? 1 : 0);
+  if (need > (size_t)DT_SDPA_STATIC_SCRATCH_BYTES) return DT_OOM;  // beyond the fixed array: use dt_sdpa_f16
+  void* ws = nullptr;
+  if (need > 0) {
+    if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
+    ws = sdpa_static_scratch();
+    if (!ws) return DT_DEVICE_ERROR;
+  }
+  return sdpa_enqueue(stream, B, Hq, Hk, D, n_qseg, q_seg, n_kvseg, k_seg, v_seg, rot_q, rot_k, eps, o, scale, Wo, bo,
+                      ws, need);
 }

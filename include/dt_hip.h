@@ -310,6 +310,29 @@ dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32
 size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int64_t Sq,
                                int64_t Skv, int32_t fused_prep, int32_t fused_out_proj);
 
+/*
+ * dt_sdpa_f16 with the library's own scratch instead of a caller's workspace.  No counterpart in the reference:
+ * it exists for callers that cannot allocate device memory around the call -- code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  Same arguments, validation, kernels and results as dt_sdpa_f16;
+ * it calls nothing that allocates or frees.
+ *   The scratch is one fixed array of DT_SDPA_STATIC_SCRATCH_BYTES per GPU, resident on every GPU the library runs
+ *   on until the process ends (its device address is looked up once per device, by dt_init or by the first call
+ *   with that device current).  A request whose dt_sdpa_workspace_bytes() exceeds it returns DT_OOM and enqueues
+ *   nothing: use dt_sdpa_f16 with a workspace of the caller's then.  The limit covers the fused QK-norm / RoPE
+ *   staging of a joint sequence of 4608 tokens x 24 heads x 128 (56.6 MB) and the fused unify-heads staging of
+ *   SD 1.5 (5.2 MB).
+ *   All calls on one GPU share that GPU's array, whose contents are whatever the last call left (every byte a
+ *   call reads it has written first): calls that may overlap in time on one GPU -- different streams, or different
+ *   threads -- race on it and must be ordered by the caller.  Calls on one stream are ordered by the stream.
+ */
+#define DT_SDPA_STATIC_SCRATCH_BYTES (64u << 20)
+
+dt_status dt_sdpa_f16_static(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D,
+                             int32_t n_qseg, const dt_seq_segment* q_seg, int32_t n_kvseg,
+                             const dt_seq_segment* k_seg, const dt_seq_segment* v_seg,
+                             const uint16_t* rot_q, const uint16_t* rot_k, float eps, dt_view4 o,
+                             float scale, const uint16_t* Wo, const uint16_t* bo);
+
 #ifdef __cplusplus
 }
 #endif
