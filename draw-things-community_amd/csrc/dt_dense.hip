@@ -10,7 +10,7 @@
 //
 // Tile: BM x BN outputs per 512-thread workgroup (8 waves, two per SIMD, each
 // a BN/2 x BM/4 slice), K-tiles of 32 processed in pairs; one barrier per K-tile.
-#include "dt_dense_kernel.h"
+#include "dt_dense_launch.h"
 
 namespace dt {
 

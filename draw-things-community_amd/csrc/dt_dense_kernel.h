@@ -145,6 +145,309 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
 }
 
+// ---- epilogue, shared by the tiled kernels -------------------------------------------------------------------
+// acc: the wave's WN x WM slice as TN x TM blocks of 32 x 32 (rows = features, columns = tokens).  nw / mw: first
+// feature (inside weight w) and first token of the slice; m_total: rows of X.  smem: the workgroup's LDS, free
+// for reuse (the caller's K loop ended with a barrier); the wave parks its slice at smem + wave * WM * WN halfs.
+template <int WN, int WM, bool POST>
+__device__ __forceinline__ void dense_epilogue(float16_t (&acc)[WN / 32][WM / 32], unsigned char* smem, int wave, int lane,
+                                               int nw, int64_t mw, const DenseWeight& w, int m_total) {
+  constexpr int TN = WN / 32, TM = WM / 32;
+  const int l32 = lane & 31, hi = lane >> 5;
+  const bool head = WN == 128 && !POST && (w.gamma || w.rot);
+  // ---- epilogue --------------------------------------------------------------
+  // The K loop ended with a barrier, so its LDS tiles are free.  Every wave parks
+  // its WN x WM slice -- bias added, rounded to fp16: the Dense's own result -- in
+  // its own part of LDS as [token][feature] rows and then walks it row by row in a
+  // short loop: RPI token rows per trip, CH lanes of 8 consecutive features per
+  // row, so that every access to memory is a whole 16-byte chunk of a row (32 bytes
+  // for the fp32 stream) and the code stays small (a fully unrolled walk over the
+  // accumulators spends most of its time fetching instructions: measured 47 us per
+  // workgroup for the GELU tail, against 7 us for this form).  The tails -- per-head
+  // RMSNorm + RoPE, or scale / addend / activation / gate / residual -- run in that
+  // loop, rounding to fp16 wherever the separate ops would; a plain Dense just
+  // stores the parked rows.
+  constexpr int CH = WN / 8;    // 16-byte chunks per parked row
+  constexpr int RPI = 64 / CH;  // token rows per trip
+  half_t* const park = reinterpret_cast<half_t*>(smem) + wave * (WM * WN);
+  {
+    // Accumulator block (i, j): lane holds token (lane & 31) of the block and
+    // features 8 g + 4 (lane / 32) + (0..3), g = 0..3.  Chunk c of token t is
+    // parked at chunk c ^ (t % CH): the 8-byte writes of 32 tokens spread over the banks.
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+      for (int gq = 0; gq < 4; gq++) {
+        const int nn = nw + i * 32 + 8 * gq + 4 * hi;
+        float b4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (w.bias) {
+          if (nn + 3 < w.n && (reinterpret_cast<uintptr_t>(w.bias) & 7) == 0) {
+            const uint2_t bb = *reinterpret_cast<const uint2_t*>(w.bias + nn);
+            b4[0] = (float)bits_to_half((uint16_t)bb[0]);
+            b4[1] = (float)bits_to_half((uint16_t)(bb[0] >> 16));
+            b4[2] = (float)bits_to_half((uint16_t)bb[1]);
+            b4[3] = (float)bits_to_half((uint16_t)(bb[1] >> 16));
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              if (nn + e < w.n) b4[e] = (float)bits_to_half(w.bias[nn + e]);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < TM; j++) {
+          const int t = j * 32 + l32;
+          const uint2_t pk = {pack_h2(acc[i][j][4 * gq] + b4[0], acc[i][j][4 * gq + 1] + b4[1]),
+                              pack_h2(acc[i][j][4 * gq + 2] + b4[2], acc[i][j][4 * gq + 3] + b4[3])};
+          *reinterpret_cast<uint2_t*>(park + t * WN + (((i * 4 + gq) ^ (t & (CH - 1))) << 3) + 4 * hi) = pk;
+        }
+      }
+  }
+  // a wave's LDS operations execute in order: its reads below see the writes above
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  const int c = lane & (CH - 1), rsub = lane / CH;
+  const int nn = nw + 8 * c;    // first of this lane's 8 features
+  if (nw >= w.n) return;
+  // this lane's column data
+  float gt[8];  // the gate, or the RMSNorm weight of a head tile
+#pragma unroll
+  for (int e = 0; e < 8; e++) gt[e] = 1.f;
+  auto lo16 = [](uint32_t v) { return (float)bits_to_half((uint16_t)v); };
+  auto hi16 = [](uint32_t v) { return (float)bits_to_half((uint16_t)(v >> 16)); };
+  if (head && w.gamma) {
+    if ((reinterpret_cast<uintptr_t>(w.gamma) & 15) == 0) {
+      const uint4_t gg = *reinterpret_cast<const uint4_t*>(w.gamma + 8 * c);
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        gt[2 * q] = lo16(gg[q]);
+        gt[2 * q + 1] = hi16(gg[q]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) gt[e] = (float)bits_to_half(w.gamma[8 * c + e]);
+    }
+  }
+  if constexpr (POST) {
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      if (nn + e < w.n) {
+        if (w.gate) gt[e] = (float)bits_to_half(w.gate[nn + e]);
+        if (w.gate32) gt[e] = w.gate32[nn + e];
+      }
+  }
+  // what a row needs from memory before its arithmetic
+  struct RowIn {
+    uint4_t add;  // the addend, or the RoPE table row of a head tile
+    uint4_t mul;
+    float4_t r0, r1;
+  };
+  // FAST: the wave's slice lies inside the matrix and every row meets the vector alignment
+  // ACT: the activation when it is known where the loop is instantiated (the fast form is instantiated once
+  // per activation, so that its body holds one activation's code), or -1 = taken from the arguments at run time
+  auto walk = [&](auto fast_tag, auto act_tag) {
+    constexpr bool FAST = decltype(fast_tag)::value;
+    constexpr int ACT = decltype(act_tag)::value;
+    auto fetch = [&](int it, RowIn& in) {
+      const int t = it * RPI + rsub;
+      const int64_t gm = mw + t;
+      if (head && w.rot) in.add = *reinterpret_cast<const uint4_t*>(w.rot + (w.rot_pos0 + gm) * WN + 8 * c);
+      if constexpr (POST) {
+        if (w.add) in.add = *reinterpret_cast<const uint4_t*>(w.add + gm * w.ld_add + nn);
+        if (w.mul) in.mul = *reinterpret_cast<const uint4_t*>(w.mul + gm * w.ld_mul + nn);
+        if (w.res) {
+          in.r0 = *reinterpret_cast<const float4_t*>(w.res + gm * w.ld_res + nn);
+          in.r1 = *reinterpret_cast<const float4_t*>(w.res + gm * w.ld_res + nn + 4);
+        }
+      }
+    };
+    // Trips go in groups of GRP: the rows a group needs from memory are requested one group ahead, before the
+    // previous group's stores (a load behind a store waits for it), so a trip does not wait a memory round trip.
+    constexpr int TRIPS = WM / RPI;
+    constexpr int GRP = (FAST && !POST) ? 4 : 1;
+    static_assert(TRIPS % GRP == 0, "trips per group");
+    RowIn cur[GRP];
+    if constexpr (FAST) {
+#pragma unroll
+      for (int j = 0; j < GRP; j++) fetch(j, cur[j]);
+    }
+    for (int it0 = 0; it0 < TRIPS; it0 += GRP) {
+      RowIn nxt[GRP];
+      if constexpr (FAST) {
+        if (it0 + GRP < TRIPS) {
+#pragma unroll
+          for (int j = 0; j < GRP; j++) fetch(it0 + GRP + j, nxt[j]);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < GRP; j++) {
+      const int it = it0 + j;
+      const int t = it * RPI + rsub;
+      const int64_t gm = mw + t;
+      const bool row_ok = FAST || gm < m_total;
+      const int64_t gmc = row_ok ? gm : 0;
+      const uint4_t raw = *reinterpret_cast<const uint4_t*>(park + t * WN + ((c ^ (t & (CH - 1))) << 3));
+      float v[8] = {lo16(raw[0]), hi16(raw[0]), lo16(raw[1]), hi16(raw[1]),
+                    lo16(raw[2]), hi16(raw[2]), lo16(raw[3]), hi16(raw[3])};
+      float res[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (head) {
+        // per-head RMSNorm and RoPE: a parked row is one head, spread over the CH = 16 lanes of a DPP row
+        if (w.gamma) {
+          float ss = 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; e++) ss += v[e] * v[e];
+          ss = row16_sum(ss);
+          const float inv = 1.0f / sqrtf(ss / (float)WN + w.eps);
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = round_f16(v[e] * inv * gt[e]);
+        }
+        if (w.rot) {
+          uint4_t rr;
+          if constexpr (FAST) {
+            rr = cur[j].add;
+          } else {
+            const uint16_t* rrow = w.rot + (w.rot_pos0 + gmc) * WN + 8 * c;
+#pragma unroll
+            for (int q = 0; q < 4; q++) rr[q] = (uint32_t)rrow[2 * q] | ((uint32_t)rrow[2 * q + 1] << 16);
+          }
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const float cs = lo16(rr[q]), sn = hi16(rr[q]);
+            const float re = v[2 * q], im = v[2 * q + 1];
+            v[2 * q] = round_f16(re * cs - im * sn);
+            v[2 * q + 1] = round_f16(re * sn + im * cs);
+          }
+        }
+      }
+      if constexpr (POST) {
+        float ad[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (w.add) {
+          if constexpr (FAST) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              ad[2 * q] = lo16(cur[j].add[q]);
+              ad[2 * q + 1] = hi16(cur[j].add[q]);
+            }
+          } else if (row_ok) {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              if (nn + e < w.n) ad[e] = (float)bits_to_half(w.add[gmc * w.ld_add + nn + e]);
+          }
+        }
+        float ml[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
+        if (w.mul) {
+          if constexpr (FAST) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              ml[2 * q] = lo16(cur[j].mul[q]);
+              ml[2 * q + 1] = hi16(cur[j].mul[q]);
+            }
+          } else if (row_ok) {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              if (nn + e < w.n) ml[e] = (float)bits_to_half(w.mul[gmc * w.ld_mul + nn + e]);
+          }
+        }
+        if (w.res) {
+          if constexpr (FAST) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              res[e] = cur[j].r0[e];
+              res[4 + e] = cur[j].r1[e];
+            }
+          } else if (row_ok) {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              if (nn + e < w.n) res[e] = w.res[gmc * w.ld_res + nn + e];
+          }
+        }
+        // post_value's steps, each over the row's 8 values under one uniform test (a step that is off costs a
+        // branch, not eight selects)
+        const auto rh = [](float x) { return round_f16(x); };
+        if (w.scale != 1.0f) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(v[e] * w.scale);
+        }
+        if (w.add) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(v[e] + ad[e]);
+        }
+        if (w.mul) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(v[e] * ml[e]);
+        }
+        const int act = ACT >= 0 ? ACT : w.act;
+        if (act == DT_ACT_GELU_TANH) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(act_gelu_tanh(v[e]));
+        } else if (act == DT_ACT_SWISH) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(act_swish(v[e]));
+        } else if (act == DT_ACT_GELU_ERF) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(act_gelu_erf(v[e]));
+        }
+        if (w.gate) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = rh(v[e] * gt[e]);
+        }
+        if (w.res) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            float pr = w.gate32 ? v[e] * gt[e] : v[e];  // the fp32 gate's product is its own op: rounded before the addition
+            asm volatile("" : "+v"(pr));
+            res[e] += pr;
+          }
+        }
+      }
+      const uint4_t out = {pack_h2(v[0], v[1]), pack_h2(v[2], v[3]), pack_h2(v[4], v[5]), pack_h2(v[6], v[7])};
+      if constexpr (FAST) {
+        if constexpr (POST) {
+          if (w.res) {
+            *reinterpret_cast<float4_t*>(w.res + gm * w.ld_res + nn) = float4_t{res[0], res[1], res[2], res[3]};
+            *reinterpret_cast<float4_t*>(w.res + gm * w.ld_res + nn + 4) = float4_t{res[4], res[5], res[6], res[7]};
+          }
+        }
+        if (w.y) *reinterpret_cast<uint4_t*>(w.y + gm * w.ldy + nn) = out;
+      } else if (row_ok) {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          if (nn + e < w.n) {
+            if constexpr (POST) {
+              if (w.res) w.res[gmc * w.ld_res + nn + e] = res[e];
+            }
+            if (w.y) w.y[gmc * w.ldy + nn + e] = (uint16_t)(out[e >> 1] >> (16 * (e & 1)));
+          }
+      }
+      }
+      if constexpr (FAST) {
+#pragma unroll
+        for (int j = 0; j < GRP; j++) cur[j] = nxt[j];
+      }
+    }
+  };
+  const bool aligned16 = (!w.y || (((w.ldy & 7) == 0) && (reinterpret_cast<uintptr_t>(w.y) & 15) == 0)) &&
+                         (!(head && w.rot) || (reinterpret_cast<uintptr_t>(w.rot) & 15) == 0) &&
+                         (!POST || ((!w.add || (((w.ld_add & 7) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 15) == 0)) &&
+                                    (!w.mul || (((w.ld_mul & 7) == 0) && (reinterpret_cast<uintptr_t>(w.mul) & 15) == 0)) &&
+                                    (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0))));
+  if (aligned16 && nw + WN <= w.n && mw + WM <= m_total) {
+    if constexpr (POST) {
+      switch (w.act) {
+        case DT_ACT_GELU_TANH: walk(std::true_type{}, std::integral_constant<int, DT_ACT_GELU_TANH>{}); break;
+        case DT_ACT_SWISH: walk(std::true_type{}, std::integral_constant<int, DT_ACT_SWISH>{}); break;
+        case DT_ACT_GELU_ERF: walk(std::true_type{}, std::integral_constant<int, DT_ACT_GELU_ERF>{}); break;
+        default: walk(std::true_type{}, std::integral_constant<int, DT_ACT_NONE>{}); break;
+      }
+    } else {
+      walk(std::true_type{}, std::integral_constant<int, DT_ACT_NONE>{});
+    }
+  } else {
+    walk(std::false_type{}, std::integral_constant<int, -1>{});
+  }
+}
+
 // 512 threads = 8 waves, two per SIMD, all eight running MFMAs on a (BN/2) x
 // (BM/4) slice.  Every thread issues its share of the memory -> LDS transfer of
 // X and unpacks / looks up half a granule (16 weights) of one W row per
@@ -405,12 +708,15 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // Written as assembly, like the transfers: the closing s_waitcnt of an
   // iteration covers these stores, and the compiler has no reason to order
   // them against anything else.
-  const uint32_t w_dst = lds_address(Bs) + 2u * (uint32_t)lds_chunk(b_row, second ? 2 : 0);
+  // unpacked weight tiles are chunk-major, [4 chunks of 8 k][BN rows][8 halfs]: a wave's 64 rows of one chunk are
+  // 1 KB of consecutive addresses, for the row-per-lane writes here and for the row-per-lane operand reads alike
+  auto w_chunk = [](int row, int c) { return (c * BN + row) * 8; };
+  const uint32_t w_dst = lds_address(Bs) + 2u * (uint32_t)w_chunk(b_row, second ? 2 : 0);
   auto write_weights = [&](int stage, int h) {
     if constexpr (MODE != kPlainF16) {
       const uint4_t v = {la[8 * h] | (la[8 * h + 1] << 16), la[8 * h + 2] | (la[8 * h + 3] << 16),
                          la[8 * h + 4] | (la[8 * h + 5] << 16), la[8 * h + 6] | (la[8 * h + 7] << 16)};
-      const uint32_t addr = (w_dst + (uint32_t)(stage * B_STAGE * 2)) ^ (uint32_t)(h << 4);  // chunks c0, c0 + 1 differ in bit 4
+      const uint32_t addr = w_dst + (uint32_t)(stage * B_STAGE * 2) + (uint32_t)(h * BN * 16);
       asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
     }
   };
@@ -453,7 +759,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     if constexpr (MODE == kPlainF16)
       fw[buf][i] = *reinterpret_cast<const half8_t*>(wp + (w_lane ^ ((4 * par + 2 * ks) << 3)) + i * 32 * PROW);
     else
-      fw[buf][i] = *reinterpret_cast<const half8_t*>(Bs + stage * B_STAGE + lds_chunk(wrow + i * 32, 2 * ks + hi));
+      fw[buf][i] = *reinterpret_cast<const half8_t*>(Bs + stage * B_STAGE + ((2 * ks + hi) * BN + wrow + i * 32) * 8);
   };
   auto read_x = [&](int buf, int j, const half_t* xs, int par, int ks) {
     fx[buf][j] = *reinterpret_cast<const half8_t*>(xs + (x_lane ^ ((4 * par + 2 * ks) << 3)) + j * 32 * PROW);
@@ -603,341 +909,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     iteration(t + 1, 1, XsA, WpA, XsB, WpB);
   }
 
-  const bool head = WN == 128 && !POST && (w.gamma || w.rot);
-  // ---- epilogue --------------------------------------------------------------
-  // The K loop ended with a barrier, so its LDS tiles are free.  Every wave parks
-  // its WN x WM slice -- bias added, rounded to fp16: the Dense's own result -- in
-  // its own part of LDS as [token][feature] rows and then walks it row by row in a
-  // short loop: RPI token rows per trip, CH lanes of 8 consecutive features per
-  // row, so that every access to memory is a whole 16-byte chunk of a row (32 bytes
-  // for the fp32 stream) and the code stays small (a fully unrolled walk over the
-  // accumulators spends most of its time fetching instructions: measured 47 us per
-  // workgroup for the GELU tail, against 7 us for this form).  The tails -- per-head
-  // RMSNorm + RoPE, or scale / addend / activation / gate / residual -- run in that
-  // loop, rounding to fp16 wherever the separate ops would; a plain Dense just
-  // stores the parked rows.
-  constexpr int CH = WN / 8;    // 16-byte chunks per parked row
-  constexpr int RPI = 64 / CH;  // token rows per trip
-  half_t* const park = reinterpret_cast<half_t*>(smem) + wave * (WM * WN);
-  {
-    // Accumulator block (i, j): lane holds token (lane & 31) of the block and
-    // features 8 g + 4 (lane / 32) + (0..3), g = 0..3.  Chunk c of token t is
-    // parked at chunk c ^ (t % CH): the 8-byte writes of 32 tokens spread over the banks.
-#pragma unroll
-    for (int i = 0; i < TN; i++)
-#pragma unroll
-      for (int gq = 0; gq < 4; gq++) {
-        const int nn = n0 + wn * WN + i * 32 + 8 * gq + 4 * hi;
-        float b4[4] = {0.f, 0.f, 0.f, 0.f};
-        if (w.bias) {
-          if (nn + 3 < w.n && (reinterpret_cast<uintptr_t>(w.bias) & 7) == 0) {
-            const uint2_t bb = *reinterpret_cast<const uint2_t*>(w.bias + nn);
-            b4[0] = (float)bits_to_half((uint16_t)bb[0]);
-            b4[1] = (float)bits_to_half((uint16_t)(bb[0] >> 16));
-            b4[2] = (float)bits_to_half((uint16_t)bb[1]);
-            b4[3] = (float)bits_to_half((uint16_t)(bb[1] >> 16));
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-              if (nn + e < w.n) b4[e] = (float)bits_to_half(w.bias[nn + e]);
-          }
-        }
-#pragma unroll
-        for (int j = 0; j < TM; j++) {
-          const int t = j * 32 + l32;
-          const uint2_t pk = {pack_h2(acc[i][j][4 * gq] + b4[0], acc[i][j][4 * gq + 1] + b4[1]),
-                              pack_h2(acc[i][j][4 * gq + 2] + b4[2], acc[i][j][4 * gq + 3] + b4[3])};
-          *reinterpret_cast<uint2_t*>(park + t * WN + (((i * 4 + gq) ^ (t & (CH - 1))) << 3) + 4 * hi) = pk;
-        }
-      }
-  }
-  // a wave's LDS operations execute in order: its reads below see the writes above
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-  const int c = lane & (CH - 1), rsub = lane / CH;
-  const int nw = n0 + wn * WN;  // first feature of this wave's slice
-  const int nn = nw + 8 * c;    // first of this lane's 8 features
-  if (nw >= w.n) return;
-  // this lane's column data
-  float gt[8];  // the gate, or the RMSNorm weight of a head tile
-#pragma unroll
-  for (int e = 0; e < 8; e++) gt[e] = 1.f;
-  auto lo16 = [](uint32_t v) { return (float)bits_to_half((uint16_t)v); };
-  auto hi16 = [](uint32_t v) { return (float)bits_to_half((uint16_t)(v >> 16)); };
-  if (head && w.gamma) {
-    if ((reinterpret_cast<uintptr_t>(w.gamma) & 15) == 0) {
-      const uint4_t gg = *reinterpret_cast<const uint4_t*>(w.gamma + 8 * c);
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        gt[2 * q] = lo16(gg[q]);
-        gt[2 * q + 1] = hi16(gg[q]);
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; e++) gt[e] = (float)bits_to_half(w.gamma[8 * c + e]);
-    }
-  }
-  if constexpr (POST) {
-#pragma unroll
-    for (int e = 0; e < 8; e++)
-      if (nn + e < w.n) {
-        if (w.gate) gt[e] = (float)bits_to_half(w.gate[nn + e]);
-        if (w.gate32) gt[e] = w.gate32[nn + e];
-      }
-  }
-  // what a row needs from memory before its arithmetic
-  struct RowIn {
-    uint4_t add;  // the addend, or the RoPE table row of a head tile
-    uint4_t mul;
-    float4_t r0, r1;
-  };
-  // FAST: the wave's slice lies inside the matrix and every row meets the vector alignment
-  // ACT: the activation when it is known where the loop is instantiated (the fast form is instantiated once
-  // per activation, so that its body holds one activation's code), or -1 = taken from the arguments at run time
-  auto walk = [&](auto fast_tag, auto act_tag) {
-    constexpr bool FAST = decltype(fast_tag)::value;
-    constexpr int ACT = decltype(act_tag)::value;
-    auto fetch = [&](int it, RowIn& in) {
-      const int t = it * RPI + rsub;
-      const int64_t gm = m0 + wm * WM + t;
-      if (head && w.rot) in.add = *reinterpret_cast<const uint4_t*>(w.rot + (w.rot_pos0 + gm) * WN + 8 * c);
-      if constexpr (POST) {
-        if (w.add) in.add = *reinterpret_cast<const uint4_t*>(w.add + gm * w.ld_add + nn);
-        if (w.mul) in.mul = *reinterpret_cast<const uint4_t*>(w.mul + gm * w.ld_mul + nn);
-        if (w.res) {
-          in.r0 = *reinterpret_cast<const float4_t*>(w.res + gm * w.ld_res + nn);
-          in.r1 = *reinterpret_cast<const float4_t*>(w.res + gm * w.ld_res + nn + 4);
-        }
-      }
-    };
-    // Trips go in groups of GRP: the rows a group needs from memory are requested one group ahead, before the
-    // previous group's stores (a load behind a store waits for it), so a trip does not wait a memory round trip.
-    constexpr int TRIPS = WM / RPI;
-    constexpr int GRP = (FAST && !POST) ? 4 : 1;
-    static_assert(TRIPS % GRP == 0, "trips per group");
-    RowIn cur[GRP];
-    if constexpr (FAST) {
-#pragma unroll
-      for (int j = 0; j < GRP; j++) fetch(j, cur[j]);
-    }
-    for (int it0 = 0; it0 < TRIPS; it0 += GRP) {
-      RowIn nxt[GRP];
-      if constexpr (FAST) {
-        if (it0 + GRP < TRIPS) {
-#pragma unroll
-          for (int j = 0; j < GRP; j++) fetch(it0 + GRP + j, nxt[j]);
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < GRP; j++) {
-      const int it = it0 + j;
-      const int t = it * RPI + rsub;
-      const int64_t gm = m0 + wm * WM + t;
-      const bool row_ok = FAST || gm < g.m;
-      const int64_t gmc = row_ok ? gm : 0;
-      const uint4_t raw = *reinterpret_cast<const uint4_t*>(park + t * WN + ((c ^ (t & (CH - 1))) << 3));
-      float v[8] = {lo16(raw[0]), hi16(raw[0]), lo16(raw[1]), hi16(raw[1]),
-                    lo16(raw[2]), hi16(raw[2]), lo16(raw[3]), hi16(raw[3])};
-      float res[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      if (head) {
-        // per-head RMSNorm and RoPE: a parked row is one head, spread over the CH = 16 lanes of a DPP row
-        if (w.gamma) {
-          float ss = 0.f;
-#pragma unroll
-          for (int e = 0; e < 8; e++) ss += v[e] * v[e];
-          ss = row16_sum(ss);
-          const float inv = 1.0f / sqrtf(ss / (float)WN + w.eps);
-#pragma unroll
-          for (int e = 0; e < 8; e++) v[e] = round_f16(v[e] * inv * gt[e]);
-        }
-        if (w.rot) {
-          uint4_t rr;
-          if constexpr (FAST) {
-            rr = cur[j].add;
-          } else {
-            const uint16_t* rrow = w.rot + (w.rot_pos0 + gmc) * WN + 8 * c;
-#pragma unroll
-            for (int q = 0; q < 4; q++) rr[q] = (uint32_t)rrow[2 * q] | ((uint32_t)rrow[2 * q + 1] << 16);
-          }
-#pragma unroll
-          for (int q = 0; q < 4; q++) {
-            const float cs = lo16(rr[q]), sn = hi16(rr[q]);
-            const float re = v[2 * q], im = v[2 * q + 1];
-            v[2 * q] = round_f16(re * cs - im * sn);
-            v[2 * q + 1] = round_f16(re * sn + im * cs);
-          }
-        }
-      }
-      if constexpr (POST) {
-        float ad[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        if (w.add) {
-          if constexpr (FAST) {
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-              ad[2 * q] = lo16(cur[j].add[q]);
-              ad[2 * q + 1] = hi16(cur[j].add[q]);
-            }
-          } else if (row_ok) {
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-              if (nn + e < w.n) ad[e] = (float)bits_to_half(w.add[gmc * w.ld_add + nn + e]);
-          }
-        }
-        float ml[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
-        if (w.mul) {
-          if constexpr (FAST) {
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-              ml[2 * q] = lo16(cur[j].mul[q]);
-              ml[2 * q + 1] = hi16(cur[j].mul[q]);
-            }
-          } else if (row_ok) {
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-              if (nn + e < w.n) ml[e] = (float)bits_to_half(w.mul[gmc * w.ld_mul + nn + e]);
-          }
-        }
-        if (w.res) {
-          if constexpr (FAST) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              res[e] = cur[j].r0[e];
-              res[4 + e] = cur[j].r1[e];
-            }
-          } else if (row_ok) {
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-              if (nn + e < w.n) res[e] = w.res[gmc * w.ld_res + nn + e];
-          }
-        }
-        // post_value's steps, each over the row's 8 values under one uniform test (a step that is off costs a
-        // branch, not eight selects)
-        const auto rh = [](float x) { return round_f16(x); };
-        if (w.scale != 1.0f) {
-#pragma unroll
-          for (int e = 0; e < 8; e++) v[e] = rh(v[e] * w.scale);
-        }
-        if (w.add) {
-#pragma unroll
-          for (int e = 0; e < 8; e++) v[e] = rh(v[e] + ad[e]);
-        }
-        if (w.mul) {
-#pragma unroll
-          for (int e = 0; e < 8; e++) v[e] = rh(v[e] * ml[e]);
-        }
-        const int act = ACT >= 0 ? ACT : w.act;
-        if (act == DT_ACT_GELU_TANH) {
-#pragma unroll
-          for (int e = 0; e < 8; e++) v[e] = rh(act_gelu_tanh(v[e]));
-        } else if (act == DT_ACT_SWISH) {
-#pragma unroll
-          for (int e = 0; e < 8; e++) v[e] = rh(act_swish(v[e]));
-        } else if (act == DT_ACT_GELU_ERF) {
-#pragma unroll
-          for (int e = 0; e < 8; e++) v[e] = rh(act_gelu_erf(v[e]));
-        }
-        if (w.gate) {
-#pragma unroll
-          for (int e = 0; e < 8; e++) v[e] = rh(v[e] * gt[e]);
-        }
-        if (w.res) {
-#pragma unroll
-          for (int e = 0; e < 8; e++) {
-            float pr = w.gate32 ? v[e] * gt[e] : v[e];  // the fp32 gate's product is its own op: rounded before the addition
-            asm volatile("" : "+v"(pr));
-            res[e] += pr;
-          }
-        }
-      }
-      const uint4_t out = {pack_h2(v[0], v[1]), pack_h2(v[2], v[3]), pack_h2(v[4], v[5]), pack_h2(v[6], v[7])};
-      if constexpr (FAST) {
-        if constexpr (POST) {
-          if (w.res) {
-            *reinterpret_cast<float4_t*>(w.res + gm * w.ld_res + nn) = float4_t{res[0], res[1], res[2], res[3]};
-            *reinterpret_cast<float4_t*>(w.res + gm * w.ld_res + nn + 4) = float4_t{res[4], res[5], res[6], res[7]};
-          }
-        }
-        if (w.y) *reinterpret_cast<uint4_t*>(w.y + gm * w.ldy + nn) = out;
-      } else if (row_ok) {
-#pragma unroll
-        for (int e = 0; e < 8; e++)
-          if (nn + e < w.n) {
-            if constexpr (POST) {
-              if (w.res) w.res[gmc * w.ld_res + nn + e] = res[e];
-            }
-            if (w.y) w.y[gmc * w.ldy + nn + e] = (uint16_t)(out[e >> 1] >> (16 * (e & 1)));
-          }
-      }
-      }
-      if constexpr (FAST) {
-#pragma unroll
-        for (int j = 0; j < GRP; j++) cur[j] = nxt[j];
-      }
-    }
-  };
-  const bool aligned16 = (!w.y || (((w.ldy & 7) == 0) && (reinterpret_cast<uintptr_t>(w.y) & 15) == 0)) &&
-                         (!(head && w.rot) || (reinterpret_cast<uintptr_t>(w.rot) & 15) == 0) &&
-                         (!POST || ((!w.add || (((w.ld_add & 7) == 0) && (reinterpret_cast<uintptr_t>(w.add) & 15) == 0)) &&
-                                    (!w.mul || (((w.ld_mul & 7) == 0) && (reinterpret_cast<uintptr_t>(w.mul) & 15) == 0)) &&
-                                    (!w.res || (((w.ld_res & 3) == 0) && (reinterpret_cast<uintptr_t>(w.res) & 15) == 0))));
-  if (aligned16 && nw + WN <= w.n && m0 + wm * WM + WM <= g.m) {
-    if constexpr (POST) {
-      switch (w.act) {
-        case DT_ACT_GELU_TANH: walk(std::true_type{}, std::integral_constant<int, DT_ACT_GELU_TANH>{}); break;
-        case DT_ACT_SWISH: walk(std::true_type{}, std::integral_constant<int, DT_ACT_SWISH>{}); break;
-        case DT_ACT_GELU_ERF: walk(std::true_type{}, std::integral_constant<int, DT_ACT_GELU_ERF>{}); break;
-        default: walk(std::true_type{}, std::integral_constant<int, DT_ACT_NONE>{}); break;
-      }
-    } else {
-      walk(std::true_type{}, std::integral_constant<int, DT_ACT_NONE>{});
-    }
-  } else {
-    walk(std::false_type{}, std::integral_constant<int, -1>{});
-  }
-}
-
-
-// Tile shapes the host side chooses between.
-enum DenseTile : int { kTile128x128 = 0, kTile128x256 = 1, kTile256x256 = 2 };
-
-template <int Q, int BM, int BN, bool POST>
-static dt_status launch_tiled(hipStream_t s, const DenseArgs& a, int mode) {
-  dim3 grid((unsigned)a.total_tiles), block(512);
-  if constexpr (Q == 16) {  // plain fp16 weight
-    hipLaunchKernelGGL((dense_qx_kernel<8, BM, BN, kPlainF16, POST>), grid, block, 0, s, a);
-    return launch_status();
-  } else {
-    switch (mode) {
-      case kPalShared: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalShared, POST>), grid, block, 0, s, a); break;
-      case kPalRow:
-        if constexpr ((BN << (Q + 1)) <= kPalLdsBytes) {
-          hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalRow, POST>), grid, block, 0, s, a);
-          break;
-        } else {
-          return DT_NO_KERNEL;  // choose_pal_mode never picks per-row palettes that do not fit
-        }
-      default: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalGlobal, POST>), grid, block, 0, s, a); break;
-    }
-    return launch_status();
-  }
-}
-
-template <int Q, bool POST>
-static dt_status launch_dense_qp(hipStream_t s, const DenseArgs& a, int tile, int mode) {
-  switch (tile) {
-    case kTile128x128: return launch_tiled<Q, 128, 128, POST>(s, a, mode);
-    case kTile128x256: return launch_tiled<Q, 128, 256, POST>(s, a, mode);
-    default: return launch_tiled<Q, 256, 256, POST>(s, a, mode);
-  }
-}
-
-// Every tiled kernel for Q-bit indices (Q = 16: plain fp16 weights); `post` selects the variant with the
-// elementwise tail.  Instantiated once per Q in dt_dense_q<Q>.hip.
-template <int Q>
-dt_status launch_dense_q(hipStream_t s, const DenseArgs& a, int tile, bool post, int mode) {
-  return post ? launch_dense_qp<Q, true>(s, a, tile, mode) : launch_dense_qp<Q, false>(s, a, tile, mode);
+  dense_epilogue<WN, WM, POST>(acc, smem, wave, lane, n0 + wn * WN, (int64_t)m0 + wm * WM, w, g.m);
 }
 
 }  // namespace dt

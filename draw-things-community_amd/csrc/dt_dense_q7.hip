@@ -1,5 +1,5 @@
 // K1 instantiations for 7-bit palette indices (all tile shapes, with and without the elementwise tail).
-#include "dt_dense_kernel.h"
+#include "dt_dense_launch.h"
 
 namespace dt {
 template dt_status launch_dense_q<7>(hipStream_t, const DenseArgs&, int, bool, int);
