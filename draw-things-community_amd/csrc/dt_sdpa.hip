@@ -267,7 +267,6 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   float l_run = 0.f;        // this lane's share of the row sum
 
   const float c = PREMUL ? 1.0f : a.scale_log2e;
-  const float thr = 8.0f / c;  // rescale only when the maximum grows by more than 2^8
   const int n_tiles = (int)((Skv + BKV - 1) / BKV);
 
   float16_t sacc[2];   // S^T of the tile in flight (keys x queries)
@@ -321,14 +320,35 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
           sacc[kb][v] = s;
         }
     }
-    float mx = sacc[0][0];
+    // Probabilities against the current reference, and this lane's share of their row sum.  The tile's maximum is
+    // not looked for: as long as every lane's sum stays below 2^10 no probability exceeds that (fp16 holds 2^16),
+    // which is all that the reference is there to ensure.
+    float psum;
+    auto probabilities = [&]() __attribute__((always_inline)) {
+      const float mc = m_ref * c;
+      psum = 0.f;
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++)
+      for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-      for (int v = (kb == 0 ? 1 : 0); v < 16; v++) mx = fmaxf(mx, sacc[kb][v]);
-    mx = max32(mx);
-    if (__builtin_amdgcn_ballot_w64(mx > m_ref + thr) != 0) {
-      // some row's maximum moved far enough: move every row's reference up to its running maximum
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const float p = fast_exp2(__builtin_fmaf(sacc[kb][8 * tt + e], c, -mc));
+            psum += p;
+            pf[kb][tt][e] = (half_t)p;
+          }
+    };
+    probabilities();
+    // (the first tile arrives here with the reference at -inf: its sums are inf; a NaN fails the test too)
+    if (__builtin_amdgcn_ballot_w64(!(psum <= 1024.0f)) != 0) {
+      // some row's scores have outgrown the reference: move every row's reference up to its running maximum,
+      // rescale what has been accumulated, and redo this tile's probabilities
+      float mx = sacc[0][0];
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int v = (kb == 0 ? 1 : 0); v < 16; v++) mx = fmaxf(mx, sacc[kb][v]);
+      mx = max32(mx);
       const float m_new = fmaxf(m_ref, mx);
       const float alpha = fast_exp2((m_ref - m_new) * c);  // first tile: exp2(-inf) = 0
       m_ref = m_new;
@@ -337,19 +357,8 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       for (int db = 0; db < DB; db++)
 #pragma unroll
         for (int v = 0; v < 16; v++) oacc[db][v] *= alpha;
+      probabilities();
     }
-    const float mc = m_ref * c;
-    float psum = 0.f;
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-      for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-          const float p = fast_exp2(__builtin_fmaf(sacc[kb][8 * tt + e], c, -mc));
-          psum += p;
-          pf[kb][tt][e] = (half_t)p;
-        }
     l_run += psum;
   };
 
