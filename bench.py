@@ -23,6 +23,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
 # counters read for a 256 MiB device copy (x2.00 and x1.00); the summary is profiles/bench_flux_block_counters.txt
 MEASURED_TRAFFIC_BYTES = {"dense_qkv": 3.750e8, "sdpa": 1.326e8}
+TRAFFIC_SOURCE = "profiles/bench_flux_block_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script; not measured by this run)"
 
 
 def other_configs(pkg, torch, np):
@@ -85,6 +86,16 @@ def other_configs(pkg, torch, np):
     dense("cfg1 Dense q6p M8192 320->320", 8192, 320, [320], "q6p", 10)
     dense("cfg2 Dense q8p M4608 3072->3x3072", 4608, 3072, [3072] * 3, "q8p", 10)
     dense("cfg2 Dense q8p M4608 3072->3072", 4608, 3072, [3072], "q8p", 10)
+    # sensitivity to the palette block size (the per-codec constants are inferred from file sizes, not read from
+    # the codec's source): q6p and q8p at every candidate, same shape
+    for codec in ("q6p", "q8p"):
+        qb = pkg.CODEC[codec][0]
+        for nb in (512, 1024, 4096, 16384):
+            x = torch.randn(4608, 3072, device=dev).half()
+            ws = [synth(3072, 3072, qb, nb) for _ in range(3)]
+            outs = [torch.empty(4608, 3072, device=dev, dtype=torch.float16) for _ in range(3)]
+            record(f"cfg2 nib sweep Dense {codec} nib{nb} M4608 3072->3x3072", 2.0 * 4608 * 3072 * 9216,
+                   timed(lambda: pkg.dense_multi(x, ws, [None] * 3, outs=outs), 10))
     sdpa("cfg4 Flux 2048^2 attention H24 D128 S16896", 1, 16896, 16896, 24, 128, 3)
     dense("cfg4 Dense q4p M16896 3072->3x3072", 16896, 3072, [3072] * 3, "q4p", 3)
     sdpa("cfg5 Wan self-attention H40 D128 S32760", 1, 32760, 32760, 40, 128, 2)
@@ -93,19 +104,73 @@ def other_configs(pkg, torch, np):
     return out
 
 
+def clock_probe(pkg, torch, np, k_dense, k_sdpa, zero_inputs):
+    """What the card's clock does under the step's two kernels: each runs back to back for ~2.5 s on its normal
+    (random) inputs and again with all activations zero, while `rocm-smi --showclocks` is sampled from a second
+    thread.  Same instruction stream both times; the difference is what the data does to the card's power draw."""
+    import subprocess
+    import threading
+
+    def sclk():
+        try:
+            out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+            for line in out.splitlines():
+                if "sclk" in line and "(" in line:
+                    return int(line.split("(")[1].split("Mhz")[0])
+        except Exception:
+            return None
+        return None
+
+    res = {}
+    for kname, fn, flop in (("dense_qkv", k_dense[0], k_dense[1]), ("sdpa", k_sdpa[0], k_sdpa[1])):
+        for data in ("random", "zero"):
+            if data == "zero":
+                zero_inputs(True)
+            stop, count = [False], [0]
+
+            def spin():
+                while not stop[0]:
+                    for _ in range(50):
+                        fn()
+                    torch.cuda.synchronize()
+                    count[0] += 50
+
+            th = threading.Thread(target=spin)
+            th.start()
+            time.sleep(1.0)
+            c0, t0 = count[0], time.perf_counter()
+            clocks = []
+            for _ in range(3):
+                time.sleep(0.4)
+                clocks.append(sclk())
+            c1, t1 = count[0], time.perf_counter()
+            stop[0] = True
+            th.join()
+            if data == "zero":
+                zero_inputs(False)
+            ms = (t1 - t0) * 1e3 / max(c1 - c0, 1)
+            res[f"{kname}_{data}"] = {"sclk_mhz": clocks, "ms": round(ms, 4), "tflops": round(flop / ms / 1e9, 1)}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # One step is ~0.7 ms; the card needs ~50 ms of continuous work to reach its sustained clock, so the default
-    # warm-up is 100 steps.  Fewer than that measures the clock ramp (about 6 % slower), not the kernels.
+    # One step is ~0.7 ms.  The clock settling is taken care of by --prewarm-ms, not by these two.
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--prewarm-ms", type=float, default=150.0,
+                    help="wall time of untimed steps before the counted warm-up, so that the clock has settled "
+                         "however few warm-up steps are asked for")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch the step's kernels one by one instead of as a HIP graph")
-    ap.add_argument("--kernel-iters", type=int, default=50, help="launches per kernel for the per-kernel timings")
+    ap.add_argument("--kernel-iters", type=int, default=100, help="launches per kernel for the per-kernel timings")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--clock-probe", action="store_true",
+                    help="also run the two kernels of the step for a few seconds each on random and on all-zero "
+                         "activations while sampling the card's clock with rocm-smi (adds 'clock_probe' to the line)")
     ap.add_argument("--other-configs", action="store_true",
                     help="also time the operators of the other benchmark configurations (SD 1.5, q8p Dense alone, "
                          "Flux at 2048 x 2048 with q4p, Wan 14B with q5p) and add them to the JSON line as 'other_configs'")
@@ -262,6 +327,16 @@ def main():
             print(f"graph capture failed, running eagerly: {e}", file=sys.stderr)
             torch.cuda.synchronize()
 
+    # The card needs tens of milliseconds of continuous work before its clock settles (a cold card runs the first
+    # launches faster or slower than the sustained rate, depending on where the governor starts): run the step for
+    # --prewarm-ms of wall time first, whatever --warmup says.  The counted warm-up and the timed region follow
+    # without a gap, and the timed region is exactly --steps steps.
+    t_pre = time.perf_counter()
+    while (time.perf_counter() - t_pre) * 1e3 < args.prewarm_ms:
+        for _ in range(20):
+            run_step()
+        torch.cuda.synchronize()
+    prewarm_ms = (time.perf_counter() - t_pre) * 1e3
     for _ in range(args.warmup):
         run_step()
     torch.cuda.synchronize()
@@ -274,9 +349,14 @@ def main():
 
     # ---------------- per-kernel timings (events on the launch stream) ----------------
     def time_kernel(fn, iters):
-        for _ in range(max(2, iters // 4)):
-            fn()
+        # ~30 ms of the same kernel first: a kernel's sustained clock depends on the kernel
+        fn()
         torch.cuda.synchronize()
+        t_w = time.perf_counter()
+        while time.perf_counter() - t_w < 0.03:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(iters):
@@ -336,7 +416,8 @@ def main():
     roofline = {
         "kernel": dom, "bound": "mfma", "achieved": round(tf(dom_flop, dom_ms), 2), "peak": PEAK_F16_TFLOPS,
         "unit": "TFLOP/s", "frac": round(tf(dom_flop, dom_ms) / PEAK_F16_TFLOPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES[dom_tr], "flop_per_launch": dom_flop, "avg_launch_ms": round(dom_ms, 4),
+        "traffic": MEASURED_TRAFFIC_BYTES[dom_tr], "traffic_source": TRAFFIC_SOURCE,
+        "flop_per_launch": dom_flop, "avg_launch_ms": round(dom_ms, 4),
         "others": {
             "sdpa_kernel<128> S=4608 H=24": {"achieved": round(tf(flop_sdpa, ms["sdpa_S4608"]), 2),
                                              "frac": round(tf(flop_sdpa, ms["sdpa_S4608"]) / PEAK_F16_TFLOPS, 4),
@@ -388,10 +469,27 @@ def main():
         }
 
     other = other_configs(pkg, torch, np) if args.other_configs else None
+    probe = None
+    if args.clock_probe:
+        saved = {}
+
+        def zero_inputs(on):
+            for name, t in (("img", img), ("ctx", ctx), ("qkv", qkv)):
+                if on:
+                    saved[name] = t.clone()
+                    t.zero_()
+                else:
+                    t.copy_(saved[name])
+            torch.cuda.synchronize()
+
+        k_qkv()  # fills qkv for the attention leg
+        torch.cuda.synchronize()
+        probe = clock_probe(pkg, torch, np, (k_qkv, 2.0 * S * C * 3 * C), (k_sdpa, flop_sdpa), zero_inputs)
 
     line = {
         "metric": "SDPA + palettized-GEMM TFLOP/s (% fp16 peak); ms/block, Flux 4608 tok q6p",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "prewarm_ms": round(prewarm_ms, 1),
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic", "launch": launch_mode,
         "config": {"workload": "Flux.1-dev joint attention block hot path: 512 text + 4096 image tokens, 24x128 heads, "
@@ -402,6 +500,8 @@ def main():
     }
     if other is not None:
         line["other_configs"] = other
+    if probe is not None:
+        line["clock_probe"] = probe
     print(json.dumps(line))
 
 

@@ -80,12 +80,13 @@ static dt_status launch_dense(hipStream_t s, const DenseArgs& a, int tile, int q
 }
 
 // Palette placement for a BN-row tile (see PalMode).
-static int choose_pal_mode(int qbits, int nib, int64_t K, int BN) {
+static int choose_pal_mode(int qbits, int nib, int64_t K, int BM, int BN) {
   if (qbits == 16) return kPlainF16;
   const int64_t pal_bytes = (int64_t)2 << qbits;
-  if ((int64_t)BN * pal_bytes <= kPalLdsBytes) return kPalRow;
+  const int64_t budget = pal_lds_bytes(BM, BN);
+  if ((int64_t)BN * pal_bytes <= budget) return kPalRow;
   const int64_t shared_count = ((int64_t)BN * K) / nib + 2;
-  if (shared_count * pal_bytes <= kPalLdsBytes) return kPalShared;
+  if (shared_count * pal_bytes <= budget) return kPalShared;
   return kPalGlobal;
 }
 
@@ -275,7 +276,11 @@ static dt_status run_group(hipStream_t s, const HostGroup& h) {
       if (wj.qbits != w0.qbits || (wj.qbits != 16 && wj.nib != w0.nib) || !h.w_tiled(j)) break;
       big_tiles += ((M + 255) / 256) * ((wj.count / K + 255) / 256);
     }
-    const bool big = ((M >= 1024) && (n_rows0 >= 256) && big_tiles >= kFillTiles) || any_fused;
+    // (palettes that fit beside no big tile -- 256-entry palettes with small blocks -- would be looked up in memory:
+    // the small tile holds a per-row table of them and is several times faster, unless a fused epilogue needs the big one)
+    const bool pal_fits_big = choose_pal_mode(w0.qbits, w0.nib, K, 256, 256) != kPalGlobal ||
+                              choose_pal_mode(w0.qbits, w0.nib, K, 128, 128) == kPalGlobal;
+    const bool big = (((M >= 1024) && (n_rows0 >= 256) && big_tiles >= kFillTiles) && pal_fits_big) || any_fused;
     // few token rows: halve the token tile so that more workgroups share the work
     const bool narrow = big && M < 1024;
     const int BM = big ? (narrow ? 128 : 256) : 128, BN = big ? 256 : 128;
@@ -301,7 +306,7 @@ static dt_status run_group(hipStream_t s, const HostGroup& h) {
     if ((int64_t)g.tiles_m * tiles_n > 0x7fffffff) return DT_NO_KERNEL;
     a.total_tiles = g.tiles_m * tiles_n;
     finish_args(a, 1, cnt, K, w0);
-    const int mode = choose_pal_mode(w0.qbits, a.nib, K, BN);
+    const int mode = choose_pal_mode(w0.qbits, a.nib, K, BM, BN);
     dt_status st = launch_dense(s, a, !big ? kTile128x128 : narrow ? kTile128x256 : kTile256x256, w0.qbits, mode);
     if (st != DT_OK) return st;
     for (int j = first; j < i; j++)
@@ -332,6 +337,9 @@ static bool run_groups_fused(hipStream_t s, const HostGroup* hs, int n, dt_statu
     total_w += h.n_weights;
   }
   if (!big || total_w > kMaxWeights) return false;
+  if (choose_pal_mode(w0.qbits, w0.nib, hs[0].K, 256, 256) == kPalGlobal &&
+      choose_pal_mode(w0.qbits, w0.nib, hs[0].K, 128, 128) != kPalGlobal)
+    return false;  // problem by problem, on the small tile with its per-row palette table
   // the kernel variant with the elementwise tail has no fused head epilogue: such problems do not share a launch
   bool any_post = false, any_epi = false;
   for (int gi = 0; gi < n; gi++) {
@@ -362,7 +370,7 @@ static bool run_groups_fused(hipStream_t s, const HostGroup* hs, int n, dt_statu
   }
   a.total_tiles = (int32_t)tiles;
   finish_args(a, n, cnt, hs[0].K, w0);
-  const int mode = choose_pal_mode(w0.qbits, a.nib, hs[0].K, BN);
+  const int mode = choose_pal_mode(w0.qbits, a.nib, hs[0].K, BM, BN);
   dt_status st = launch_dense(s, a, kTile256x256, w0.qbits, mode);
   for (int gi = 0; gi < n && st == DT_OK; gi++)
     for (int i = 0; i < hs[gi].n_weights && st == DT_OK; i++)

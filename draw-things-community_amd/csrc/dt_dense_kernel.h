@@ -14,6 +14,9 @@ constexpr int kMaxWeights = 8;
 constexpr int kMaxGroups = 4;
 constexpr int BK = 32;
 constexpr int kPalLdsBytes = 32768;
+// LDS a tile shape can spare for palettes: the 128 x 128 tile's X slots and weight ring are a quarter of the
+// 256 x 256 tile's, which leaves room for a per-row table of 256-entry palettes (128 rows x 512 B).
+constexpr int pal_lds_bytes(int BM, int BN) { return (BM == 128 && BN == 128) ? 65536 : kPalLdsBytes; }
 
 enum PalMode : int {
   kPalShared = 0,  // palettes of every block the tile's rows touch, loaded once, slot = block - first block
@@ -474,7 +477,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // their addresses then fit an instruction offset.  X (and a plain fp16 W) lives in two pair slots, each
   // holding two K-tiles as [rows][64 halfs]: one is read while the next pair is in flight into the other.
   constexpr bool HAS_PAL = MODE == kPalShared || MODE == kPalRow;
-  constexpr int PAL_BYTES = HAS_PAL ? kPalLdsBytes : 0;
+  constexpr int PAL_BYTES = HAS_PAL ? pal_lds_bytes(BM, BN) : 0;
   constexpr int XS_BYTES = BM * PROW * 2;
   constexpr int WP_BYTES = MODE == kPlainF16 ? BN * PROW * 2 : 0;
   constexpr int BS_BYTES = MODE == kPlainF16 ? 0 : NST * B_STAGE * 2;

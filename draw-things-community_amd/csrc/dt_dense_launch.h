@@ -17,7 +17,7 @@ static dt_status launch_tiled(hipStream_t s, const DenseArgs& a, int mode) {
     switch (mode) {
       case kPalShared: hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalShared, POST>), grid, block, 0, s, a); break;
       case kPalRow:
-        if constexpr ((BN << (Q + 1)) <= kPalLdsBytes) {
+        if constexpr ((BN << (Q + 1)) <= pal_lds_bytes(BM, BN)) {
           hipLaunchKernelGGL((dense_qx_kernel<Q, BM, BN, kPalRow, POST>), grid, block, 0, s, a);
           break;
         } else {

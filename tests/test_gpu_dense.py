@@ -58,6 +58,9 @@ CASES = [
     (1536, 384, 256, 5, 1024),    # q5p, a palette block per four rows
     (4100, 130, 128, 4, 512),     # ragged last token tile and a two-row last feature tile
     (2048, 256, 192, 6, 64),      # the palette block changes inside a row every two K-tiles
+    (1300, 1024, 1024, 8, 4096),  # 256-entry palettes with small blocks: fit beside no big tile -> small tile, per-row table
+    (1100, 520, 768, 8, 512),     # the same with several blocks per row (K % nib != 0), ragged edges
+    (1100, 768, 512, 7, 1024),    # 128-entry palettes, two rows per block
 ]
 
 
