@@ -40,6 +40,7 @@ ABI_SYMBOLS = (
     "dt_sdpa_f16",
     "dt_sdpa_workspace_bytes",
     "dt_sdpa_f16_static",
+    "dt_lora_branch_f32_f16",
 )
 
 STATIC_SCRATCH_BYTES = 64 << 20  # DT_SDPA_STATIC_SCRATCH_BYTES
@@ -141,6 +142,8 @@ def lib():
                                   vp, vp, vp, ctypes.c_size_t]
         L.dt_sdpa_f16_static.restype = i32
         L.dt_sdpa_f16_static.argtypes = L.dt_sdpa_f16.argtypes[:-2]
+        L.dt_lora_branch_f32_f16.restype = i32
+        L.dt_lora_branch_f32_f16.argtypes = [vp, i64, i64, vp, i64, vp, i32, vp, i64, f32, vp, vp, i64]
         L.dt_sdpa_workspace_bytes.restype = ctypes.c_size_t
         L.dt_sdpa_workspace_bytes.argtypes = [i32, i32, i32, i32, i64, i64, i32, i32]
         _lib = L
@@ -538,13 +541,13 @@ class LoRADense:
     left packed and the fp16 low-rank pair applied beside it (Models/LoRA.swift:85-142; running the LoRA separately
     is the preferred mode for quantized models, Models/UNetProtocol.swift:696-697).  Three launches of the Dense
     kernel: down (with the scale in its epilogue) beside the base projection, then up, whose epilogue adds the base
-    projection's result; every intermediate is rounded to fp16 as the reference's separate ops round.  `highPrecision` (an fp32 down
-    projection) is not provided by the library."""
+    projection's result; every intermediate is rounded to fp16 as the reference's separate ops round.  With
+    `highPrecision` the pair is fp32 (`down.data` / `up.data` float32 tensors): the branch is computed as
+    fp16(up(scale * down(float(x)))) in fp32 throughout (Models/LoRA.swift:117-139) by dt_lora_branch_f32_f16 and added
+    in the base projection's epilogue."""
 
     def __init__(self, count: int, configuration: LoRANetworkConfiguration, noBias: bool = False, flags: int = 0,
                  name: str = ""):
-        if configuration.highPrecision:
-            raise NotImplementedError("LoRADense: highPrecision (fp32 down projection) is not available")
         self.count, self.configuration, self.noBias, self.flags, self.name = count, configuration, noBias, flags, name
         self.weight: Optional[QxTensor] = None
         self.bias = None
@@ -587,10 +590,12 @@ class LoRADense:
             return dense_post(x, [self.weight], [b], [post], flags=self.flags, stream=stream)[0]
         if self.down.shape[0] != self.configuration.rank or self.up.shape != (self.count, self.configuration.rank):
             raise ValueError(f"LoRADense {self.name!r}: down / up shapes do not match rank and count")
-        dn, up = self._padded()
         p = post or DensePost()
         if p.scale != 1.0 or p.addend is not None or p.multiplicand is not None:
             raise ValueError(f"LoRADense {self.name!r}: the tail may carry an activation, a gate and a residual only")
+        if self.configuration.highPrecision:
+            return self._high_precision(x, b, p, stream)
+        dn, up = self._padded()
         # The down projection is a few dozen workgroups that wait on memory; the base projection does not depend on
         # it.  They go out side by side on two streams, and the up projection, whose epilogue adds the base
         # projection's result and then runs the tail, follows both.  (fp16(base) + fp16(branch) rounds the same
@@ -606,6 +611,39 @@ class LoRADense:
         out = dense_post(down, [up], [None], [tail], stream=main)[0]
         return None if out is None else out.reshape(*x.shape[:-1], self.count)
 
+
+def _lora_high_precision(self, x, b, p, stream):
+    """out = dense(x) + fp16(up32(scale * down32(float(x)))), then the tail: the fp32 branch beside the base projection
+    on a second stream, the sum in the base projection's epilogue."""
+    torch = _torch()
+    dn, up = self.down.data, self.up.data
+    if dn.dtype != torch.float32 or up.dtype != torch.float32 or not dn.is_contiguous() or not up.is_contiguous():
+        raise TypeError(f"LoRADense {self.name!r}: highPrecision takes contiguous float32 down / up weights")
+    _f16_cuda(x, "x")
+    K, r = x.shape[-1], self.configuration.rank
+    x2 = x.reshape(-1, K)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    main = stream if stream is not None else torch.cuda.current_stream(x.device)
+    side = _side_stream(x.device)
+    side.wait_stream(main)
+    with torch.cuda.stream(side):
+        T = torch.empty((M, r), dtype=torch.float32, device=x.device)
+        branch = torch.empty((M, self.count), dtype=torch.float16, device=x.device)
+        st = lib().dt_lora_branch_f32_f16(_stream_ptr(side), M, K, x2.data_ptr(), x2.stride(0), dn.data_ptr(), r,
+                                          up.data_ptr(), self.count, float(self.configuration.scale), T.data_ptr(),
+                                          branch.data_ptr(), branch.stride(0))
+        _check("dt_lora_branch_f32_f16", st)
+    main.wait_stream(side)
+    T.record_stream(main)
+    branch.record_stream(main)
+    tail = DensePost(p.activation, p.gate, p.residual, p.keep_output, addend=branch)
+    out = dense_post(x2, [self.weight], [b], [tail], flags=self.flags, stream=main)[0]
+    return None if out is None else out.reshape(*x.shape[:-1], self.count)
+
+
+LoRADense._high_precision = _lora_high_precision
 
 _SIDE_STREAMS = {}
 

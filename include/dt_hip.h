@@ -232,6 +232,19 @@ dt_status dt_layernorm_modulate_f16(dt_stream stream, int64_t M, int64_t C, cons
                                     uint16_t* Y, int64_t ldy);
 
 /*
+ * The low-rank branch of a LoRADense in high precision (LoRANetworkConfiguration.highPrecision,
+ * Models/LoRA.swift:117-139): out = fp16(up(scale * down(float(x)))) with fp32 weights, an fp32 intermediate and
+ * fp32 accumulation -- `denseDown(x.to(.Float32))`, `denseUp(configuration.scale * downX).to(of: x)`.  The caller
+ * adds it to the base projection through dt_dense_post.addend (out = dense(x) + branch).
+ *   X    : [M, K] fp16, row stride ldx          down : [rank, K] fp32        up : [N, rank] fp32
+ *   T    : scratch for the intermediate, [M, rank] fp32
+ *   out  : [M, N] fp16, row stride ldo
+ */
+dt_status dt_lora_branch_f32_f16(dt_stream stream, int64_t M, int64_t K, const uint16_t* X, int64_t ldx,
+                                 const float* down, int32_t rank, const float* up, int64_t N, float scale,
+                                 float* T, uint16_t* out, int64_t ldo);
+
+/*
  * Several independent Dense problems (each an X with its weights, arguments as
  * for dt_dense_qx_heads_f16) enqueued together.  The context (text) and image
  * streams of a joint block apply different weights to different token sets

@@ -424,6 +424,16 @@ def np_lora_branch16(X16: np.ndarray, down16: np.ndarray, up16: np.ndarray, scal
     return np_dense64(d, up16).astype(np.float16)
 
 
+def np_lora_branch32(X16: np.ndarray, down32: np.ndarray, up32: np.ndarray, scale: float = 1.0) -> np.ndarray:
+    """The low-rank branch with highPrecision (Models/LoRA.swift:117-139): `denseDown(x.to(.Float32))`,
+    `denseUp(scale * downX).to(of: x)` -- fp32 weights and intermediate, one rounding to fp16 at the end.  Evaluated in
+    float64 and rounded to fp32 where the graph holds fp32 tensors (the fp32 GEMMs' own summation error, ~1e-6
+    relative, is below what the final fp16 rounding keeps)."""
+    t = (X16.astype(np.float64) @ down32.astype(np.float64).T).astype(np.float32)
+    t = (np.float32(scale) * t).astype(np.float32)
+    return (t.astype(np.float64) @ up32.astype(np.float64).T).astype(np.float32).astype(np.float16)
+
+
 def np_add16(a16: np.ndarray, b16: np.ndarray) -> np.ndarray:
     """fp16 elementwise sum (out = dense(x) + up(...), Models/LoRA.swift:128-140); the float32 sum of two fp16 values
     is exact, so one rounding."""

@@ -763,3 +763,44 @@ def test_operators_on_a_side_stream(dthip, oracle, torch_cuda):
     want_o = oracle.C.sdpa(want_z[None], want_z[None], x, 1 / np.sqrt(D))
     mx, rr = oracle.err_stats(o.cpu().numpy(), want_o)
     assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+@pytest.mark.parametrize("M,N,K,q,nib,rank,scale", [(300, 512, 256, 6, 4096, 16, 1.0), (1100, 384, 192, 4, 512, 64, 0.5),
+                                                     (70, 100, 96, 16, 0, 8, 2.0), (4608, 3072, 3072, 6, 4096, 32, 0.75)])
+def test_lora_dense_high_precision(dthip, oracle, torch_cuda, M, N, K, q, nib, rank, scale):
+    """LoRADense with highPrecision: the low-rank pair is fp32 and the branch fp16(up(scale * down(float(x)))) is
+    computed in fp32 throughout (Models/LoRA.swift:117-139).  The branch against float64 (one fp16 ulp, or 2^-16 of the
+    row's largest entry where cancellation leaves less), the sum bit for bit on the device's own base and branch."""
+    torch = torch_cuda
+    rng = np.random.default_rng(M + rank)
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    if q == 16:
+        Wh = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+        w = dthip.QxTensor.from_f16(Wh)
+    else:
+        w, _ = make_weight(dthip, oracle, rng, N, K, q, nib, std=0.05)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float16)
+    down = (rng.standard_normal((rank, K)) * 0.1).astype(np.float32)
+    up = (rng.standard_normal((N, rank)) * 0.1).astype(np.float32)
+    xd, bd = to_dev(torch, X), to_dev(torch, bias)
+    print("lora dense high precision", M, N, K, q, rank, scale, flush=True)
+    layer = dthip.LoRADense(N, dthip.LoRANetworkConfiguration(rank, scale, highPrecision=True))
+    layer.weight, layer.bias = w, bd
+    layer.down = dthip.QxTensor(to_dev(torch, down), 32, 0, down.shape)
+    layer.up = dthip.QxTensor(to_dev(torch, up), 32, 0, up.shape)
+    out = layer(xd).cpu().numpy()
+    # the branch alone, through the C ABI
+    T = torch.empty((M, rank), dtype=torch.float32, device="cuda")
+    br = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    st = dthip.lib().dt_lora_branch_f32_f16(None, M, K, xd.data_ptr(), K, layer.down.data.data_ptr(), rank,
+                                            layer.up.data.data_ptr(), N, scale, T.data_ptr(), br.data_ptr(), N)
+    assert st == 0
+    got, want = br.cpu().numpy().astype(np.float64), oracle.np_lora_branch32(X, down, up, scale).astype(np.float64)
+    tol = np.maximum(np.abs(want) * 2.0 ** -10, np.abs(want).max(axis=1, keepdims=True) * 2.0 ** -16) + 2.0 ** -24
+    assert np.all(np.abs(got - want) <= tol), float(np.max(np.abs(got - want) / tol))
+    base = dthip.dense_multi(xd, [w], [bd])[0].cpu().numpy()
+    assert np.array_equal(out.view(np.uint16), oracle.np_add16(base, br.cpu().numpy()).view(np.uint16))
+    # with a tail behind the sum
+    g = layer(xd, post=dthip.DensePost(dthip.ACT_GELU_TANH))
+    o = dthip.dense_post(xd, [w], [bd], [dthip.DensePost(dthip.ACT_GELU_TANH, addend=br)])[0]
+    assert torch.equal(g, o)
