@@ -22,7 +22,7 @@ PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
 # counters read for a 256 MiB device copy (x2.00 and x1.00); the summary is profiles/bench_flux_block_counters.txt
-MEASURED_TRAFFIC_BYTES = {"dense_qkv": 3.750e8, "sdpa": 1.326e8}
+MEASURED_TRAFFIC_BYTES = {"dense_qkv": 3.742e8, "sdpa": 1.326e8}
 TRAFFIC_SOURCE = "profiles/bench_flux_block_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script; not measured by this run)"
 
 
@@ -104,10 +104,11 @@ def other_configs(pkg, torch, np):
     return out
 
 
-def clock_probe(pkg, torch, np, k_dense, k_sdpa, zero_inputs):
-    """What the card's clock does under the step's two kernels: each runs back to back for ~2.5 s on its normal
-    (random) inputs and again with all activations zero, while `rocm-smi --showclocks` is sampled from a second
-    thread.  Same instruction stream both times; the difference is what the data does to the card's power draw."""
+def clock_probe(torch, legs, zero_inputs):
+    """What the card's clock does under the step's two kernels, and under the vendor library's plain fp16 GEMM of the
+    QKV shape for comparison: each leg (name, launch, flop) runs back to back for ~2.5 s on its normal (random)
+    inputs and again with all activations zero, while `rocm-smi --showclocks` is sampled from a second thread.
+    Same instruction stream both times; the difference is what the data does to the card's power draw."""
     import subprocess
     import threading
 
@@ -122,7 +123,7 @@ def clock_probe(pkg, torch, np, k_dense, k_sdpa, zero_inputs):
         return None
 
     res = {}
-    for kname, fn, flop in (("dense_qkv", k_dense[0], k_dense[1]), ("sdpa", k_sdpa[0], k_sdpa[1])):
+    for kname, fn, flop in legs:
         for data in ("random", "zero"):
             if data == "zero":
                 zero_inputs(True)
@@ -169,7 +170,7 @@ def main():
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--clock-probe", action="store_true",
-                    help="also run the two kernels of the step for a few seconds each on random and on all-zero "
+                    help="also run the two kernels of the step, the plain fp16 Dense and the vendor library's fp16 GEMM of the QKV shape for a few seconds each on random and on all-zero "
                          "activations while sampling the card's clock with rocm-smi (adds 'clock_probe' to the line)")
     ap.add_argument("--other-configs", action="store_true",
                     help="also time the operators of the other benchmark configurations (SD 1.5, q8p Dense alone, "
@@ -349,12 +350,13 @@ def main():
 
     # ---------------- per-kernel timings (events on the launch stream) ----------------
     def time_kernel(fn, iters):
-        # ~30 ms of the same kernel first: a kernel's sustained clock depends on the kernel
+        # ~120 ms of the same kernel first: the clock the card sustains depends on the kernel, and after a lighter
+        # kernel (or an idle gap) it takes the power controller tens of milliseconds to come down to it
         fn()
         torch.cuda.synchronize()
         t_w = time.perf_counter()
-        while time.perf_counter() - t_w < 0.03:
-            for _ in range(10):
+        while time.perf_counter() - t_w < 0.12:
+            for _ in range(50):
                 fn()
             torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -473,8 +475,15 @@ def main():
     if args.clock_probe:
         saved = {}
 
+        # the library's GEMM (torch.matmul) and this library's plain fp16 Dense on the QKV shape, one problem
+        xm = torch.randn(S, C, device=dev).half()
+        wm = (torch.randn(3 * C, C, device=dev) * 0.02).half()
+        om = torch.empty(S, 3 * C, device=dev, dtype=torch.float16)
+        wq16 = [pkg.QxTensor.from_f16(wm[i * C:(i + 1) * C].contiguous()) for i in range(3)]
+        om3 = [torch.empty(S, C, device=dev, dtype=torch.float16) for _ in range(3)]
+
         def zero_inputs(on):
-            for name, t in (("img", img), ("ctx", ctx), ("qkv", qkv)):
+            for name, t in (("img", img), ("ctx", ctx), ("qkv", qkv), ("xm", xm)):
                 if on:
                     saved[name] = t.clone()
                     t.zero_()
@@ -484,7 +493,11 @@ def main():
 
         k_qkv()  # fills qkv for the attention leg
         torch.cuda.synchronize()
-        probe = clock_probe(pkg, torch, np, (k_qkv, 2.0 * S * C * 3 * C), (k_sdpa, flop_sdpa), zero_inputs)
+        flop_qkv = 2.0 * S * C * 3 * C
+        probe = clock_probe(torch, (
+            ("dense_qkv", k_qkv, flop_qkv), ("sdpa", k_sdpa, flop_sdpa),
+            ("dense_plain_f16_qkv_shape", lambda: pkg.dense_multi(xm, wq16, [None] * 3, outs=om3), flop_qkv),
+            ("library_matmul_f16_qkv_shape", lambda: torch.matmul(xm, wm.t(), out=om), flop_qkv)), zero_inputs)
 
     line = {
         "metric": "SDPA + palettized-GEMM TFLOP/s (% fp16 peak); ms/block, Flux 4608 tok q6p",
