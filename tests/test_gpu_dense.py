@@ -571,8 +571,6 @@ def test_dense_post_bad_args(dthip, oracle, torch_cuda):
         dthip.dense_post(x, [w], [None], [dthip.DensePost(addend=torch.zeros((4, 32), dtype=torch.float16, device="cuda"))])
     with pytest.raises(dthip.DtError):
         dthip.dense_post(x, [w], [None], [dthip.DensePost(scale=float("inf"))])
-    with pytest.raises(NotImplementedError):
-        dthip.LoRADense(64, dthip.LoRANetworkConfiguration(4, highPrecision=True))
 
 
 def test_dense_flux_2048_q4p_full_size_sampled(dthip, oracle, torch_cuda):
