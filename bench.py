@@ -388,6 +388,11 @@ def main():
     # the op in front of the block's Dense layers: LayerNorm + adaLN modulation of the fp32 stream (HBM-bound)
     ms["layernorm_modulate"] = time_kernel(lambda: pkg.layernorm_modulate(x32, ln_scale, ln_shift, 1e-6, out=ln_out), max(it, 10))
 
+    # the palettized format on its own: one 3072 x 3072 q6p weight to fp16 (HBM-bound byte work)
+    deq_out = torch.empty((C, C), dtype=torch.float16, device=dev)
+    ms["depalettize"] = time_kernel(lambda: w["x_o"].dequantize(out=deq_out), max(it, 10))
+    deq_bytes = len(packed_host["x_o"]) + 2 * C * C
+
     tf = lambda flop, t_ms: flop / (t_ms * 1e-3) / 1e12
     kernels = {
         "sdpa_S4608": {"ms": ms["sdpa_S4608"], "tflops": tf(flop_sdpa, ms["sdpa_S4608"]),
@@ -403,6 +408,8 @@ def main():
         "layernorm_modulate_M4608_C3072": {"ms": ms["layernorm_modulate"], "gbs": 6 * S * C / (ms["layernorm_modulate"] * 1e-3) / 1e9,
                                            "frac_hbm_peak": 6 * S * C / (ms["layernorm_modulate"] * 1e-3) / 8e12},
     }
+    kernels["depalettize_q6p_3072x3072"] = {"ms": ms["depalettize"], "gbs": deq_bytes / (ms["depalettize"] * 1e-3) / 1e9,
+                                            "frac_hbm_peak": deq_bytes / (ms["depalettize"] * 1e-3) / 8e12}
     for k in kernels.values():
         if "tflops" in k:
             k["frac_f16_peak"] = k["tflops"] / PEAK_F16_TFLOPS

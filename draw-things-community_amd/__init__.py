@@ -309,13 +309,18 @@ class QxTensor:
         w = w.to(device).contiguous()
         return QxTensor(w, 16, 0, tuple(w.shape))
 
-    def dequantize(self, stream=None):
-        """fp16 [out, in] tensor (K0): what a CPU read of the same key followed by Tensor<Float16>(from:) holds."""
+    def dequantize(self, stream=None, out=None):
+        """fp16 [out, in] tensor (K0): what a CPU read of the same key followed by Tensor<Float16>(from:) holds.
+        `out`: a contiguous fp16 tensor of that shape to fill instead of a new one."""
         torch = _torch()
         with _on(stream):
             if self.qbits == 16:
-                return self.data.clone()
-            out = torch.empty(self.shape, dtype=torch.float16, device=self.data.device)
+                return self.data.clone() if out is None else out.copy_(self.data)
+            if out is None:
+                out = torch.empty(self.shape, dtype=torch.float16, device=self.data.device)
+            elif (out.dtype != torch.float16 or tuple(out.shape) != tuple(self.shape) or not out.is_contiguous()
+                  or out.device != self.data.device):
+                raise ValueError("out must be a contiguous fp16 tensor of the weight's shape on its device")
             w = self._c()
             _check("dt_depalettize_f16", lib().dt_depalettize_f16(_stream_ptr(stream), ctypes.byref(w), out.data_ptr()))
             return out
