@@ -309,6 +309,10 @@ dt_status dt_qk_norm_rope_f16(dt_stream stream, dt_view4 x, int32_t B, int64_t S
  *   workspace : device scratch of at least dt_sdpa_workspace_bytes(...) bytes,
  *             256-byte aligned; may be NULL when that function returns 0
  * D in {40, 64, 128} (any D <= 128 that is a multiple of 8).
+ * Inputs are expected to be finite.  A key whose V row holds Inf or NaN makes every output row of its (batch,
+ * head) non-finite in the reference too, except where its probability underflows to zero; here such a V row can
+ * in addition reach rows through the unused slots of the ragged last key tile (probability exactly 0 there, and
+ * 0 x Inf = NaN).  Non-finite Q / K scores behave as in the reference (the row's output is NaN).
  */
 dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D,
                       int32_t n_qseg, const dt_seq_segment* q_seg, int32_t n_kvseg,
