@@ -28,7 +28,7 @@ def make_weight(dthip, oracle, rng, N, K, q, nib, std=0.02):
 
 
 @pytest.mark.parametrize("q", [4, 5, 6, 7, 8])
-@pytest.mark.parametrize("nib", [32, 512, 4096, 24])
+@pytest.mark.parametrize("nib", [32, 512, 1024, 4096, 16384, 24])
 def test_depalettize_bit_exact(dthip, oracle, torch_cuda, q, nib):
     torch = torch_cuda
     rng = np.random.default_rng(q * 1000 + nib)
