@@ -92,7 +92,8 @@ def test_sdpa_random_shapes(dthip, oracle, torch_cuda):
 
 def test_norm_rope_random_shapes(dthip, oracle, torch_cuda):
     """In place on a view that starts `off` elements into each row of a wider buffer.  A rotated pair is compared on
-    the scale of the pair's magnitude (the rotation keeps it; a component can cancel to far less): one fp16 ulp."""
+    the scale of the pair's magnitude (the rotation keeps it; a component can cancel to far less): one fp16 ulp per
+    stage (norm, rotation)."""
     torch = torch_cuda
     rng = np.random.default_rng(103)
     for i in range(N_CASES):
@@ -122,7 +123,10 @@ def test_norm_rope_random_shapes(dthip, oracle, torch_cuda):
                 w = oracle.C.cmul(w, rot[3:3 + S])
             wf = w.astype(np.float32)
             mag = np.sqrt(wf[..., 0::2] ** 2 + wf[..., 1::2] ** 2)
-            tol = np.repeat(np.maximum(mag * 2.0 ** -10, 2.0 ** -14), 2, axis=-1)
+            # one fp16 ulp per stage: where the normalised value lies on a rounding tie (to within the fp32 evaluation)
+            # the device and the oracle may round it apart, and the rotation carries that ulp into its result
+            stages = 2.0 if (use_g and use_r) else 1.0
+            tol = np.repeat(np.maximum(mag * 2.0 ** -10, 2.0 ** -14), 2, axis=-1) * stages
             diff = np.abs(got[b, :, off:].reshape(S, H, D).astype(np.float32) - wf)
             assert (diff <= tol).all(), (i, float((diff / tol).max()))
 
