@@ -24,6 +24,9 @@ PEAK_HBM_GBS = 8000.0
 # counters read for a 256 MiB device copy (x2.00 and x1.00); the summary is profiles/bench_flux_block_counters.txt
 MEASURED_TRAFFIC_BYTES = {"dense_qkv": 3.742e8, "sdpa": 1.326e8}
 TRAFFIC_SOURCE = "profiles/bench_flux_block_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script; not measured by this run)"
+SDPA_NAME = "sdpa_kernel<128> S=4608 H=24"
+QKV_NAME = "dense_qx_kernel<6,256,256> M=4096+512 N=3x3072 K=3072 (fused norm/RoPE epilogue)"
+OUT_NAME = "dense_qx_kernel<6,256,256> M=4096+512 N=3072 K=3072 (out projections)"
 
 
 def other_configs(pkg, torch, np):
@@ -154,6 +157,62 @@ def clock_probe(torch, legs, zero_inputs):
     return res
 
 
+class SclkSampler:
+    """Samples the card's shader clock from sysfs (pp_dpm_sclk of the PCI device torch reports for cuda:0; the
+    starred level is the current one) every few milliseconds on a thread of its own, between start() and stop()."""
+
+    def __init__(self, torch):
+        self.path = None
+        self.samples = []
+        self._stop = False
+        self._thread = None
+        try:
+            p = torch.cuda.get_device_properties(0)
+            bdf = f"{p.pci_domain_id:04x}:{p.pci_bus_id:02x}:{p.pci_device_id:02x}.0"
+            cand = f"/sys/bus/pci/devices/{bdf}/pp_dpm_sclk"
+            if os.path.exists(cand) and self._read(cand) is not None:
+                self.path = cand
+        except Exception:
+            self.path = None
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                for line in f:
+                    if "*" in line:
+                        return int(line.split(":")[1].lower().split("mhz")[0])
+        except Exception:
+            return None
+        return None
+
+    def start(self):
+        if self.path is None:
+            return
+        import threading
+
+        self._stop = False
+
+        def run():
+            while not self._stop:
+                v = self._read(self.path)
+                if v is not None:
+                    self.samples.append(v)
+                time.sleep(0.004)
+
+        self._thread = threading.Thread(target=run, daemon=True)
+        self._thread.start()
+
+    def stop(self):
+        self._stop = True
+        if self._thread is not None:
+            self._thread.join()
+        if not self.samples:
+            return None
+        xs = sorted(self.samples)
+        return {"source": self.path, "n": len(xs), "min": xs[0], "median": xs[len(xs) // 2], "max": xs[-1]}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -164,7 +223,10 @@ def main():
                     help="wall time of untimed steps before the counted warm-up, so that the clock has settled "
                          "however few warm-up steps are asked for")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-graph", action="store_true", help="launch the step's kernels one by one instead of as a HIP graph")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay the step's three kernels as a HIP graph in the timed region (default: eager launches "
+                         "with an event between them, which is no slower on this driver stack and yields the "
+                         "per-kernel times from the timed region itself)")
     ap.add_argument("--kernel-iters", type=int, default=100, help="launches per kernel for the per-kernel timings")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
@@ -248,11 +310,6 @@ def main():
             dict(x=ctx, weights=[w["c_q"], w["c_k"], w["c_v"]], biases=[bias["c_q"], bias["c_k"], bias["c_v"]],
                  outs=views(0, T), epilogues=epi_c)])
 
-    def k_prep():
-        for t4, gc, gx in ((q4, gamma["c_q"], gamma["x_q"]), (k4, gamma["c_k"], gamma["x_k"])):
-            pkg.qk_norm_rope_(t4[:, :T], gc, 1e-6, True, rot=rot, rot_pos0=0)
-            pkg.qk_norm_rope_(t4[:, T:], gx, 1e-6, True, rot=rot, rot_pos0=T)
-
     def k_sdpa():
         pkg.sdpa_segments([q4], [k4], [v4], scale, out=att)
 
@@ -284,14 +341,26 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # The step is three dependent launches; replayed as a HIP graph they go out without host gaps.  The graph is
-    # used only if its replays, with eager work in between, reproduce the eager outputs bit for bit, and only if
-    # a short trial shows it no slower than launching the three kernels one by one.
-    run_step, launch_mode = step, "eager"
-    if not args.no_graph:
+    # What the step leaves in its buffers, for the checks below: every single-kernel leg must run on the step's own
+    # data (a kernel timed on operands that another leg has degraded -- e.g. Q / K after thousands of in-place
+    # normalisation passes -- draws less power, clocks higher and reads faster than it runs in the step).
+    step()
+    torch.cuda.synchronize()
+    sig_ref = {"qkv": float(qkv.float().abs().mean()), "att": float(att.float().abs().mean())}
+
+    def check_step_inputs(leg):
+        torch.cuda.synchronize()
+        for name, t in (("qkv", qkv), ("att", att)):
+            got = float(t.float().abs().mean())
+            assert abs(got - sig_ref[name]) <= 0.1 * sig_ref[name], \
+                f"{leg}: {name} no longer holds the step's data (mean |x| {got:.4f}, after the step {sig_ref[name]:.4f})"
+
+    # The step is three dependent launches.  By default they go out one by one, with an event between them, so that
+    # the timed region itself yields the per-kernel times; --graph replays them as a HIP graph instead (then the
+    # per-kernel times come from a second, eager region of the same length right after the timed one).
+    run_step, launch_mode, graph = step, "eager (3 launches, events between them)", None
+    if args.graph:
         try:
-            step()
-            torch.cuda.synchronize()
             want = (out_x.clone(), out_c.clone(), att.clone())
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
@@ -310,28 +379,48 @@ def main():
                 step()  # eager work between replays
                 torch.cuda.synchronize()
             if ok:
-                # replays cost a little more per kernel than eager launches on some driver stacks: keep the quicker
-                def quick(fn, n=60):
-                    for _ in range(n):
-                        fn()
-                    torch.cuda.synchronize()
-                    t = time.perf_counter()
-                    for _ in range(n):
-                        fn()
-                    torch.cuda.synchronize()
-                    return time.perf_counter() - t
-                t_graph, t_eager = quick(graph.replay), quick(step)
-                t_graph, t_eager = min(t_graph, quick(graph.replay)), min(t_eager, quick(step))
-                if t_graph <= t_eager:
-                    run_step, launch_mode = graph.replay, "hip graph (3 kernels)"
+                run_step, launch_mode = graph.replay, "hip graph (3 kernels)"
+            else:
+                print("graph replays do not reproduce the eager outputs: running eagerly", file=sys.stderr)
         except Exception as e:  # capture not possible: stay eager
             print(f"graph capture failed, running eagerly: {e}", file=sys.stderr)
             torch.cuda.synchronize()
+
+    names3 = ("dense_qkv", "sdpa", "dense_out")
+
+    def step_with_events(ev):
+        ev[0].record()
+        k_qkv()
+        ev[1].record()
+        k_sdpa()
+        ev[2].record()
+        k_out()
+        ev[3].record()
+
+    def in_step_times(events):
+        """Per-kernel means over a region of eager steps with an event before and after each launch (events on the
+        launch stream), and the region's length per step from its first to its last event."""
+        acc = [0.0, 0.0, 0.0]
+        for ev in events:
+            for i in range(3):
+                acc[i] += ev[i].elapsed_time(ev[i + 1])
+        n = max(len(events), 1)
+        per = {names3[i]: acc[i] / n for i in range(3)}
+        span = events[0][0].elapsed_time(events[-1][3]) / n if events else 0.0
+        return per, span
+
+    def make_events(n):
+        return [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(n)]
 
     # The card needs tens of milliseconds of continuous work before its clock settles (a cold card runs the first
     # launches faster or slower than the sustained rate, depending on where the governor starts): run the step for
     # --prewarm-ms of wall time first, whatever --warmup says.  The counted warm-up and the timed region follow
     # without a gap, and the timed region is exactly --steps steps.
+    warm_events = make_events(1)
+    step_with_events(warm_events[0])  # first use of timing events: not measured
+    torch.cuda.synchronize()
+    events = make_events(args.steps)
+    sampler = SclkSampler(torch)
     t_pre = time.perf_counter()
     while (time.perf_counter() - t_pre) * 1e3 < args.prewarm_ms:
         for _ in range(20):
@@ -341,14 +430,28 @@ def main():
     for _ in range(args.warmup):
         run_step()
     torch.cuda.synchronize()
+    sampler.start()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run_step()
+    if graph is None or run_step is step:
+        for ev in events:
+            step_with_events(ev)
+    else:
+        for _ in range(args.steps):
+            run_step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / max(args.steps, 1)
+    if run_step is not step:
+        # the graph's replays carry no events: the breakdown comes from an eager region right behind the timed one
+        for ev in events:
+            step_with_events(ev)
+        torch.cuda.synchronize()
+    sclk = sampler.stop()
     value = flop_block / (ms_per_step * 1e-3) / 1e12
+    in_step, span_ms = in_step_times(events)
+    in_step_sum = sum(in_step.values())
+    check_step_inputs("after the timed region")
 
-    # ---------------- per-kernel timings (events on the launch stream) ----------------
+    # ---------------- single-kernel legs (events on the launch stream, back-to-back launches) ----------------
     def time_kernel(fn, iters):
         # ~120 ms of the same kernel first: the clock the card sustains depends on the kernel, and after a lighter
         # kernel (or an idle gap) it takes the power controller tens of milliseconds to come down to it
@@ -367,16 +470,25 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / iters
 
+    # the standalone norm / RoPE pass works in place: it gets a copy of Q and K of its own, never the step's buffer
+    qkv_prep = qkv.clone()
+    qp4, kp4 = qkv_prep[:, 0].unsqueeze(0), qkv_prep[:, 1].unsqueeze(0)
+
+    def k_prep():
+        for t4, gc, gx in ((qp4, gamma["c_q"], gamma["x_q"]), (kp4, gamma["c_k"], gamma["x_k"])):
+            pkg.qk_norm_rope_(t4[:, :T], gc, 1e-6, True, rot=rot, rot_pos0=0)
+            pkg.qk_norm_rope_(t4[:, T:], gx, 1e-6, True, rot=rot, rot_pos0=T)
+
     it = args.kernel_iters
-    time_kernel(k_sdpa, 2)  # first use of timing events: not measured
-    ms = {
-        "dense_qkv_grouped": time_kernel(k_qkv, it),
-        "dense_qkv_image_M4096": time_kernel(k_qkv_image, it),
-        "dense_qkv_text_M512": time_kernel(k_qkv_text, it),
-        "qk_norm_rope": time_kernel(k_prep, it),  # the standalone pass; not part of the step (fused into the QKV epilogue)
-        "sdpa_S4608": time_kernel(k_sdpa, it),
-        "dense_out_2x": time_kernel(k_out, it),
-    }
+    ms = {}
+    ms["dense_qkv_grouped"] = time_kernel(k_qkv, it)
+    ms["dense_qkv_image_M4096"] = time_kernel(k_qkv_image, it)
+    ms["dense_qkv_text_M512"] = time_kernel(k_qkv_text, it)
+    check_step_inputs("before the attention leg")  # the three legs above rewrite qkv with the step's own values
+    ms["sdpa_S4608"] = time_kernel(k_sdpa, it)
+    check_step_inputs("before the out-projection leg")
+    ms["dense_out_2x"] = time_kernel(k_out, it)
+    ms["qk_norm_rope"] = time_kernel(k_prep, it)  # the standalone pass; not part of the step (fused into the QKV epilogue)
     # the "palettized Dense alone" shape of the headline benchmark: M = 4608, 3072 -> 9216 (three weights) and 3072 -> 3072
     ms["dense_qkv_M4608_N9216"] = time_kernel(
         lambda: pkg.dense_multi(x_all, [w["x_q"], w["x_k"], w["x_v"]], [bias["x_q"], bias["x_k"], bias["x_v"]], outs=y3), it)
@@ -392,87 +504,124 @@ def main():
     deq_out = torch.empty((C, C), dtype=torch.float16, device=dev)
     ms["depalettize"] = time_kernel(lambda: w["x_o"].dequantize(out=deq_out), max(it, 10))
     deq_bytes = len(packed_host["x_o"]) + 2 * C * C
+    check_step_inputs("after the single-kernel legs")
 
     tf = lambda flop, t_ms: flop / (t_ms * 1e-3) / 1e12
-    kernels = {
-        "sdpa_S4608": {"ms": ms["sdpa_S4608"], "tflops": tf(flop_sdpa, ms["sdpa_S4608"]),
+    flop_qkv, flop_out = 2.0 * S * C * 3 * C, 2.0 * S * C * C
+    # in-step figures: what each of the step's three launches took inside the timed region
+    kernels_in_step = {
+        "dense_qkv (context + image in one launch, norm / RoPE epilogue)": {"ms": in_step["dense_qkv"], "tflops": tf(flop_qkv, in_step["dense_qkv"])},
+        "sdpa_S4608": {"ms": in_step["sdpa"], "tflops": tf(flop_sdpa, in_step["sdpa"]),
                        "ref_units_G": pkg.ScaledDotProductAttentionInstructionCount(1, H, D, S, S) / 1e9},
-        "dense_qkv_M4608_N9216_q6p": {"ms": ms["dense_qkv_M4608_N9216"], "tflops": tf(2.0 * S * C * 3 * C, ms["dense_qkv_M4608_N9216"])},
-        "dense_out_M4608_N3072_q6p": {"ms": ms["dense_out_M4608_N3072"], "tflops": tf(2.0 * S * C * C, ms["dense_out_M4608_N3072"])},
-        "dense_plainf16_M4608_N3072": {"ms": ms["dense_plainf16_M4608_N3072"], "tflops": tf(2.0 * S * C * C, ms["dense_plainf16_M4608_N3072"])},
+        "dense_out (context + image in one launch)": {"ms": in_step["dense_out"], "tflops": tf(flop_out, in_step["dense_out"])},
+    }
+    # single-kernel legs: the same launch repeated back to back (a different clock and cache state than in the step)
+    kernels = {
+        "sdpa_S4608": {"ms": ms["sdpa_S4608"], "tflops": tf(flop_sdpa, ms["sdpa_S4608"])},
+        "dense_qkv_M4608_N9216_q6p": {"ms": ms["dense_qkv_M4608_N9216"], "tflops": tf(flop_qkv, ms["dense_qkv_M4608_N9216"])},
+        "dense_out_M4608_N3072_q6p": {"ms": ms["dense_out_M4608_N3072"], "tflops": tf(flop_out, ms["dense_out_M4608_N3072"])},
+        "dense_plainf16_M4608_N3072": {"ms": ms["dense_plainf16_M4608_N3072"], "tflops": tf(flop_out, ms["dense_plainf16_M4608_N3072"])},
         "dense_qkv_image_M4096": {"ms": ms["dense_qkv_image_M4096"], "tflops": tf(2.0 * HW * C * 3 * C, ms["dense_qkv_image_M4096"])},
         "dense_qkv_text_M512": {"ms": ms["dense_qkv_text_M512"], "tflops": tf(2.0 * T * C * 3 * C, ms["dense_qkv_text_M512"])},
-        "dense_qkv_text+image_one_launch": {"ms": ms["dense_qkv_grouped"], "tflops": tf(2.0 * S * C * 3 * C, ms["dense_qkv_grouped"])},
-        "dense_out_text+image_one_launch": {"ms": ms["dense_out_2x"], "tflops": tf(2.0 * S * C * C, ms["dense_out_2x"])},
+        "dense_qkv_text+image_one_launch": {"ms": ms["dense_qkv_grouped"], "tflops": tf(flop_qkv, ms["dense_qkv_grouped"])},
+        "dense_out_text+image_one_launch": {"ms": ms["dense_out_2x"], "tflops": tf(flop_out, ms["dense_out_2x"])},
         "qk_norm_rope": {"ms": ms["qk_norm_rope"], "gbs": 2 * 2 * S * C * 2 / (ms["qk_norm_rope"] * 1e-3) / 1e9},
         "layernorm_modulate_M4608_C3072": {"ms": ms["layernorm_modulate"], "gbs": 6 * S * C / (ms["layernorm_modulate"] * 1e-3) / 1e9,
                                            "frac_hbm_peak": 6 * S * C / (ms["layernorm_modulate"] * 1e-3) / 8e12},
     }
     kernels["depalettize_q6p_3072x3072"] = {"ms": ms["depalettize"], "gbs": deq_bytes / (ms["depalettize"] * 1e-3) / 1e9,
                                             "frac_hbm_peak": deq_bytes / (ms["depalettize"] * 1e-3) / 8e12}
-    for k in kernels.values():
-        if "tflops" in k:
-            k["frac_f16_peak"] = k["tflops"] / PEAK_F16_TFLOPS
-        k["ms"] = round(k["ms"], 4)
+    for grp in (kernels, kernels_in_step):
+        for k in grp.values():
+            if "tflops" in k:
+                k["frac_f16_peak"] = round(k["tflops"] / PEAK_F16_TFLOPS, 4)
+                k["tflops"] = round(k["tflops"], 2)
+            k["ms"] = round(k["ms"], 4)
 
-    # dominant kernel of the step (by time): roofline against the fp16 MFMA peak
-    dense_ms = ms["dense_qkv_grouped"] + ms["dense_out_2x"]
-    if ms["sdpa_S4608"] >= ms["dense_qkv_grouped"]:
-        dom, dom_flop, dom_ms, dom_tr = "sdpa_kernel<128> S=4608 H=24", flop_sdpa, ms["sdpa_S4608"], "sdpa"
+    # dominant kernel of the step (the longest of its three launches, by the in-step times): roofline against the
+    # fp16 MFMA peak, algorithmic FLOPs / mean launch duration inside the timed region
+    if in_step["sdpa"] >= in_step["dense_qkv"]:
+        dom, dom_flop, dom_ms, dom_tr = SDPA_NAME, flop_sdpa, in_step["sdpa"], "sdpa"
     else:
-        dom, dom_flop, dom_ms, dom_tr = ("dense_qx_kernel<6,256,256> M=4096+512 N=3x3072 K=3072 (fused norm/RoPE epilogue)",
-                                          2.0 * S * C * 3 * C, ms["dense_qkv_grouped"], "dense_qkv")
+        dom, dom_flop, dom_ms, dom_tr = QKV_NAME, flop_qkv, in_step["dense_qkv"], "dense_qkv"
     roofline = {
         "kernel": dom, "bound": "mfma", "achieved": round(tf(dom_flop, dom_ms), 2), "peak": PEAK_F16_TFLOPS,
         "unit": "TFLOP/s", "frac": round(tf(dom_flop, dom_ms) / PEAK_F16_TFLOPS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES[dom_tr], "traffic_source": TRAFFIC_SOURCE,
         "flop_per_launch": dom_flop, "avg_launch_ms": round(dom_ms, 4),
+        "timing": "mean over the timed region's steps of the time between the events before and after the launch",
         "others": {
-            "sdpa_kernel<128> S=4608 H=24": {"achieved": round(tf(flop_sdpa, ms["sdpa_S4608"]), 2),
-                                             "frac": round(tf(flop_sdpa, ms["sdpa_S4608"]) / PEAK_F16_TFLOPS, 4),
-                                             "traffic": MEASURED_TRAFFIC_BYTES["sdpa"]},
-            "dense_qx_kernel<6,256,256> QKV, context + image in one launch": {
-                "achieved": round(tf(2.0 * S * C * 3 * C, ms["dense_qkv_grouped"]), 2),
-                "frac": round(tf(2.0 * S * C * 3 * C, ms["dense_qkv_grouped"]) / PEAK_F16_TFLOPS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES["dense_qkv"]},
+            SDPA_NAME: {"achieved": round(tf(flop_sdpa, in_step["sdpa"]), 2),
+                        "frac": round(tf(flop_sdpa, in_step["sdpa"]) / PEAK_F16_TFLOPS, 4),
+                        "avg_launch_ms": round(in_step["sdpa"], 4), "traffic": MEASURED_TRAFFIC_BYTES["sdpa"]},
+            QKV_NAME: {"achieved": round(tf(flop_qkv, in_step["dense_qkv"]), 2),
+                       "frac": round(tf(flop_qkv, in_step["dense_qkv"]) / PEAK_F16_TFLOPS, 4),
+                       "avg_launch_ms": round(in_step["dense_qkv"], 4), "traffic": MEASURED_TRAFFIC_BYTES["dense_qkv"]},
+            OUT_NAME: {"achieved": round(tf(flop_out, in_step["dense_out"]), 2),
+                       "frac": round(tf(flop_out, in_step["dense_out"]) / PEAK_F16_TFLOPS, 4),
+                       "avg_launch_ms": round(in_step["dense_out"], 4), "traffic": None},
         },
     }
 
-    # ---------------- CPU baseline: the oracle on a bounded sample ----------------
+    # ---------------- CPU baseline: the oracle on the step's own inputs, which also checks the step ----------------
     cpu = None
+    step_checked = None
     if not args.no_cpu:
         from oracle import oracle
 
         oracle.build()
         ncores = oracle.C.lib.dto_num_threads()
-        # the whole block at full size: 8 Dense (6 QKV + 2 out, per-stream rows) + attention over all heads
-        t0 = time.perf_counter()
-        xs_c = rng.standard_normal((T, C)).astype(np.float16)
-        xs_x = rng.standard_normal((HW, C)).astype(np.float16)
-        qs = rng.standard_normal((1, S, H, D)).astype(np.float16)
-        ks = rng.standard_normal((1, S, H, D)).astype(np.float16)
-        vs = rng.standard_normal((1, S, H, D)).astype(np.float16)
+        # the GPU's outputs for these inputs, from a fresh pass
+        step()
+        torch.cuda.synchronize()
+        got = {"x": out_x.cpu().numpy(), "c": out_c.cpu().numpy()}
+        host = lambda t: t.cpu().numpy()
+        xs = {"c": host(ctx), "x": host(img)}
+        bias_h = {n: host(b) for n, b in bias.items()}
+        gam_h = {n: host(g) for n, g in gamma.items()}
+        rot_h = host(rot)
+        # the whole block at full size: 8 Dense (6 QKV + 2 out, per-stream rows) + attention over all heads; the
+        # first pass keeps its outputs and is compared with the GPU's, further passes (until ~12 s of CPU work) only
+        # add to the timing
         t_dense = t_sdpa = 0.0
         passes = 0
-        while passes < 8 and t_dense + t_sdpa < 12.0:  # whole blocks until ~12 s of CPU work
+        while passes < 8 and t_dense + t_sdpa < 12.0:
             t0 = time.perf_counter()
-            for name in ("c_q", "c_k", "c_v", "c_o"):
-                oracle.C.dense_qx(xs_c, packed_host[name], qbits, nib, C, None)
-            for name in ("x_q", "x_k", "x_v", "x_o"):
-                oracle.C.dense_qx(xs_x, packed_host[name], qbits, nib, C, None)
+            proj = {s_ + n: oracle.C.dense_qx(xs[s_], packed_host[f"{s_}_{n}"], qbits, nib, C, bias_h[f"{s_}_{n}"])
+                    for s_ in "cx" for n in "qkv"}
             t1 = time.perf_counter()
-            oracle.C.sdpa(qs, ks, vs, scale)
-            t_sdpa += time.perf_counter() - t1
-            t_dense += t1 - t0
+            heads = lambda a: a.reshape(-1, H, D)
+            rq = oracle.C.cmul(np.concatenate([oracle.C.rmsnorm(heads(proj["cq"]), gam_h["c_q"], 1e-6),
+                                               oracle.C.rmsnorm(heads(proj["xq"]), gam_h["x_q"], 1e-6)]), rot_h)
+            rk = oracle.C.cmul(np.concatenate([oracle.C.rmsnorm(heads(proj["ck"]), gam_h["c_k"], 1e-6),
+                                               oracle.C.rmsnorm(heads(proj["xk"]), gam_h["x_k"], 1e-6)]), rot_h)
+            rv = np.concatenate([heads(proj["cv"]), heads(proj["xv"])])
+            t2 = time.perf_counter()
+            ratt = oracle.C.sdpa(rq[None], rk[None], rv[None], scale).reshape(S, C)
+            t3 = time.perf_counter()
+            want_c = oracle.C.dense_qx(np.ascontiguousarray(ratt[:T]), packed_host["c_o"], qbits, nib, C, bias_h["c_o"])
+            want_x = oracle.C.dense_qx(np.ascontiguousarray(ratt[T:]), packed_host["x_o"], qbits, nib, C, bias_h["x_o"])
+            t4 = time.perf_counter()
+            t_dense += (t1 - t0) + (t4 - t3)
+            t_sdpa += t3 - t2
+            if passes == 0:
+                mx_c, rr_c = oracle.err_stats(got["c"], want_c)
+                mx_x, rr_x = oracle.err_stats(got["x"], want_x)
+                step_checked = {"max_abs": round(float(max(mx_c, mx_x)), 6), "rel_rms": round(float(max(rr_c, rr_x)), 7),
+                                "bar": {"max_abs": 2e-2, "rel_rms": 2e-3},
+                                "what": "out_x [4096, 3072] and out_c [512, 3072] of the step, every element, against the "
+                                        "oracle's op-by-op pass over the same inputs and weights (Dense -> per-head "
+                                        "RMSNorm -> cmul -> two-pass softmax attention -> Dense)"}
+                step_checked["ok"] = bool(step_checked["max_abs"] <= 2e-2 and step_checked["rel_rms"] <= 2e-3)
             passes += 1
         t_dense /= passes
         t_sdpa /= passes
         t_block = t_dense + t_sdpa
         cpu = {
             "value": round(flop_block / t_block / 1e12, 5), "unit": "TFLOP/s", "cores": int(ncores), "kind": "port",
-            "sample": f"oracle (C, OpenMP, {ncores} threads), the whole block at full size, mean of {passes} passes: 8 q6p Dense "
-                      f"3072->3072 (512 / 4096 rows, depalettize included, {t_dense:.2f} s) + attention 24 heads x 4608 x 4608 "
-                      f"({t_sdpa:.2f} s); RMSNorm/RoPE not included",
+            "sample": f"oracle (C, OpenMP, {ncores} threads), the whole block at full size on the step's own inputs, mean of "
+                      f"{passes} passes: 8 q6p Dense 3072->3072 (512 / 4096 rows, depalettize included, {t_dense:.2f} s) + "
+                      f"attention 24 heads x 4608 x 4608 ({t_sdpa:.2f} s); RMSNorm/RoPE run but not timed",
             "ms_per_block": round(t_block * 1e3, 1),
             "dense_gflops": round(flop_dense / t_dense / 1e9, 1), "sdpa_gflops": round(flop_sdpa / t_sdpa / 1e9, 1),
         }
@@ -506,6 +655,7 @@ def main():
             ("dense_plain_f16_qkv_shape", lambda: pkg.dense_multi(xm, wq16, [None] * 3, outs=om3), flop_qkv),
             ("library_matmul_f16_qkv_shape", lambda: torch.matmul(xm, wm.t(), out=om), flop_qkv)), zero_inputs)
 
+    consistent = abs(in_step_sum - ms_per_step) <= 0.03 * ms_per_step
     line = {
         "metric": "SDPA + palettized-GEMM TFLOP/s (% fp16 peak); ms/block, Flux 4608 tok q6p",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -515,8 +665,14 @@ def main():
         "config": {"workload": "Flux.1-dev joint attention block hot path: 512 text + 4096 image tokens, 24x128 heads, "
                                "q6p (nib 4096) weights; 6 QKV Dense (QK RMSNorm/RoPE fused in the epilogue) + SDPA + 2 out-proj Dense",
                    "flop_per_block": flop_block, "frac_f16_peak": round(value / PEAK_F16_TFLOPS, 4)},
-        "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels,
-        "block_ms_sum_of_kernels": round(dense_ms + ms["sdpa_S4608"], 4),
+        "roofline": roofline, "cpu_baseline": cpu,
+        "kernels_in_step": kernels_in_step,
+        "in_step_ms_sum": round(in_step_sum, 4), "in_step_ms_first_to_last_event": round(span_ms, 4),
+        "breakdown_consistent": bool(consistent),
+        "breakdown_rule": "|sum of the three in-step kernel times - ms_per_step| <= 3 % of ms_per_step",
+        "sclk_mhz_during_timed_region": sclk,
+        "step_checked": step_checked,
+        "kernels_standalone_loops": kernels,
     }
     if other is not None:
         line["other_configs"] = other

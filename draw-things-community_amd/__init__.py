@@ -313,14 +313,14 @@ class QxTensor:
         """fp16 [out, in] tensor (K0): what a CPU read of the same key followed by Tensor<Float16>(from:) holds.
         `out`: a contiguous fp16 tensor of that shape to fill instead of a new one."""
         torch = _torch()
+        if out is not None and (out.dtype != torch.float16 or tuple(out.shape) != tuple(self.shape)
+                                or not out.is_contiguous() or out.device != self.data.device):
+            raise ValueError("out must be a contiguous fp16 tensor of the weight's shape on its device")
         with _on(stream):
             if self.qbits == 16:
                 return self.data.clone() if out is None else out.copy_(self.data)
             if out is None:
                 out = torch.empty(self.shape, dtype=torch.float16, device=self.data.device)
-            elif (out.dtype != torch.float16 or tuple(out.shape) != tuple(self.shape) or not out.is_contiguous()
-                  or out.device != self.data.device):
-                raise ValueError("out must be a contiguous fp16 tensor of the weight's shape on its device")
             w = self._c()
             _check("dt_depalettize_f16", lib().dt_depalettize_f16(_stream_ptr(stream), ctypes.byref(w), out.data_ptr()))
             return out
@@ -612,6 +612,9 @@ class LoRADense:
         down = dense_post(x, [dn], [None], [DensePost(scale=self.configuration.scale)], stream=side)[0]
         base = dense_multi(x, [self.weight], [b], flags=self.flags, stream=main)[0]
         main.wait_stream(side)  # every use of x and `down` on the side stream is ordered before what follows on `main`
+        # `down` came from the side stream's pool and is read on `main`: its memory must not go back to that pool's
+        # next user before `main` has passed this point
+        down.record_stream(main)
         tail = DensePost(p.activation, p.gate, p.residual, p.keep_output, addend=base.reshape(-1, self.count))
         out = dense_post(down, [up], [None], [tail], stream=main)[0]
         return None if out is None else out.reshape(*x.shape[:-1], self.count)
@@ -626,11 +629,12 @@ def _lora_high_precision(self, x, b, p, stream):
         raise TypeError(f"LoRADense {self.name!r}: highPrecision takes contiguous float32 down / up weights")
     _f16_cuda(x, "x")
     K, r = x.shape[-1], self.configuration.rank
-    x2 = x.reshape(-1, K)
-    if x2.stride(-1) != 1:
-        x2 = x2.contiguous()
-    M = x2.shape[0]
     main = stream if stream is not None else torch.cuda.current_stream(x.device)
+    with _on(main):  # a copy, if the view needs one, belongs on the caller's stream
+        x2 = x.reshape(-1, K)
+        if x2.stride(-1) != 1:
+            x2 = x2.contiguous()
+    M = x2.shape[0]
     side = _side_stream(x.device)
     side.wait_stream(main)
     with torch.cuda.stream(side):

@@ -9,12 +9,38 @@ namespace dt {
 
 constexpr int kMaxDevices = 64;
 
+// Errors after which the device (or the process's use of it) is gone: a faulted kernel, a lost or torn-down context.
+// The runtime keeps reporting these whatever is called next.
+static bool fatal_error(hipError_t e) {
+  switch (e) {
+    case hipErrorIllegalAddress:
+    case hipErrorLaunchFailure:
+    case hipErrorLaunchTimeOut:
+    case hipErrorPriorLaunchFailure:
+    case hipErrorAssert:
+    case hipErrorECCNotCorrectable:
+    case hipErrorDeinitialized:
+    case hipErrorContextIsDestroyed:
+    case hipErrorNoDevice:
+    case hipErrorUnknown:
+    case hipErrorRuntimeMemory:
+    case hipErrorRuntimeOther: return true;
+    default: return false;
+  }
+}
+
 dt_status device_ready() {
   // per device ordinal: 0 = unknown, 1 = gfx950, 2 = other
   static std::atomic<int> state[kMaxDevices];
-  // (hipErrorNotReady is the answer of a stream or event query, not a failure)
-  if (const hipError_t pending = hipPeekAtLastError(); pending != hipSuccess && pending != hipErrorNotReady)
-    return DT_DEVICE_ERROR;  // not ours: left for its owner
+  if (const hipError_t pending = hipPeekAtLastError(); pending != hipSuccess) {
+    // A fault of earlier work stays where it is, for its owner to read, and nothing is enqueued on top of it.
+    if (fatal_error(pending)) return DT_DEVICE_ERROR;
+    // Anything else in the thread's slot (a rejected argument, a pointer-attribute probe on host memory, peer
+    // access enabled twice, an unsupported query, a stream query's "not ready") is the result of a call that has
+    // already handed that code to its caller.  It is cleared so that the status read after this entry point's launch
+    // belongs to that launch.
+    (void)hipGetLastError();
+  }
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     (void)hipGetLastError();  // this query's own failure

@@ -19,15 +19,16 @@ typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
 
 namespace dt {
 
-// DT_OK when the calling thread's current device is a gfx950 part (cached per device ordinal) and the runtime holds
-// no earlier error; DT_NO_KERNEL for any other architecture; DT_DEVICE_ERROR when an error is already pending on
-// the runtime (a fault of earlier work, the caller's or anyone's: it is left in place for its owner to read, and
-// nothing is enqueued on top of it).
+// DT_OK when the calling thread's current device is a gfx950 part (cached per device ordinal); DT_NO_KERNEL for any
+// other architecture; DT_DEVICE_ERROR when the runtime already reports a fault (a kernel that faulted, a lost
+// device or context: it is left in place for its owner to read, and nothing is enqueued on top of it).  A stale
+// non-fatal code in the thread's error slot -- one that some earlier call already returned to its caller -- is
+// cleared, so that launch_status() reads this entry point's own launch.
 dt_status device_ready();
 
 inline hipStream_t as_stream(dt_stream s) { return reinterpret_cast<hipStream_t>(s); }
 
-// Result of the launch just made.  device_ready() has established that no error was pending before it, so what
+// Result of the launch just made.  device_ready() has left the thread's error slot empty, so what
 // hipGetLastError() returns here belongs to this launch: a configuration the device cannot run (grid, block, LDS or
 // register budget, missing code object) is the library's own "no kernel for this request"; bad arguments are
 // DT_INVALID; anything else (the device was lost, an asynchronous fault surfaced in between) is DT_DEVICE_ERROR.

@@ -34,13 +34,19 @@ DT_EXPORT size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int3
 
 namespace dt {
 
-// Validation and enqueue shared by dt_sdpa_f16 (caller's workspace) and dt_sdpa_f16_static (the library's own
-// per-device array).  Calls nothing that allocates.
-static dt_status sdpa_enqueue(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D, int32_t n_qseg,
-                              const dt_seq_segment* q_seg, int32_t n_kvseg, const dt_seq_segment* k_seg,
-                              const dt_seq_segment* v_seg, const uint16_t* rot_q, const uint16_t* rot_k, float eps,
-                              dt_view4 o, float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
-                              size_t workspace_bytes) {
+// What the argument checks of an attention request establish.
+struct SdpaShape {
+  int64_t Sq = 0, Skv = 0;
+  bool prep = false;   // some segment is normalised or rotated on the way in
+  bool empty = false;  // nothing to compute (no batch or no query row)
+  size_t need = 0;     // staging bytes, by the rule of dt_sdpa_workspace_bytes
+};
+
+// Argument checks shared by dt_sdpa_f16 and dt_sdpa_f16_static; touches no device state.
+static dt_status sdpa_validate(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int32_t n_qseg,
+                               const dt_seq_segment* q_seg, int32_t n_kvseg, const dt_seq_segment* k_seg,
+                               const dt_seq_segment* v_seg, const uint16_t* rot_q, const uint16_t* rot_k,
+                               const dt_view4& o, const uint16_t* Wo, SdpaShape& sh) {
   if (B < 0 || Hq <= 0 || Hk <= 0 || D <= 0 || Hq % Hk != 0) return DT_INVALID;
   if (n_qseg <= 0 || n_kvseg <= 0 || !q_seg || !k_seg || !v_seg) return DT_INVALID;
   if (n_qseg > kMaxSeg || n_kvseg > kMaxSeg) return DT_NO_KERNEL;
@@ -57,7 +63,13 @@ static dt_status sdpa_enqueue(dt_stream stream, int32_t B, int32_t Hq, int32_t H
     Skv += k_seg[i].len;
     prep = prep || k_seg[i].gamma;
   }
-  if (B == 0 || Sq == 0) return DT_OK;
+  sh.Sq = Sq;
+  sh.Skv = Skv;
+  sh.prep = prep;
+  if (B == 0 || Sq == 0) {
+    sh.empty = true;
+    return DT_OK;
+  }
   if (Skv == 0) return DT_INVALID;  // softmax over an empty set
   for (int i = 0; i < n_qseg; i++)
     if (q_seg[i].len > 0 && !view_ok(q_seg[i].view, 8)) return DT_INVALID;
@@ -65,11 +77,23 @@ static dt_status sdpa_enqueue(dt_stream stream, int32_t B, int32_t Hq, int32_t H
     if (k_seg[i].len > 0 && (!view_ok(k_seg[i].view, 8) || !view_ok(v_seg[i].view, 8))) return DT_INVALID;
   if (!o.ptr || (reinterpret_cast<uintptr_t>(o.ptr) & 7) || o.stride_b % 4 || o.stride_s % 4) return DT_INVALID;
   if (!Wo && o.stride_h % 4) return DT_INVALID;
+  sh.need = dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, prep ? 1 : 0, Wo ? 1 : 0);
+  return DT_OK;
+}
+
+// Enqueue of a request that sdpa_validate() has accepted.  Calls nothing that allocates.
+static dt_status sdpa_enqueue(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D, int32_t n_qseg,
+                              const dt_seq_segment* q_seg, int32_t n_kvseg, const dt_seq_segment* k_seg,
+                              const dt_seq_segment* v_seg, const uint16_t* rot_q, const uint16_t* rot_k, float eps,
+                              dt_view4 o, float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
+                              size_t workspace_bytes, const SdpaShape& sh) {
+  const int64_t Sq = sh.Sq, Skv = sh.Skv;
+  const bool prep = sh.prep;
+  if (sh.empty) return DT_OK;
   if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
 
-  const size_t need = dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, prep ? 1 : 0, Wo ? 1 : 0);
-  if (need > 0) {
-    if (!workspace || workspace_bytes < need) return DT_OOM;
+  if (sh.need > 0) {
+    if (!workspace || workspace_bytes < sh.need) return DT_OOM;
     if (reinterpret_cast<uintptr_t>(workspace) & 255) return DT_INVALID;
   }
   hipStream_t s = as_stream(stream);
@@ -242,8 +266,12 @@ DT_EXPORT dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t
                                 const dt_seq_segment* v_seg, const uint16_t* rot_q, const uint16_t* rot_k, float eps,
                                 dt_view4 o, float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
                                 size_t workspace_bytes) {
+  dt::SdpaShape sh;
+  if (const dt_status st = dt::sdpa_validate(B, Hq, Hk, D, n_qseg, q_seg, n_kvseg, k_seg, v_seg, rot_q, rot_k, o, Wo, sh);
+      st != DT_OK)
+    return st;
   return dt::sdpa_enqueue(stream, B, Hq, Hk, D, n_qseg, q_seg, n_kvseg, k_seg, v_seg, rot_q, rot_k, eps, o, scale, Wo,
-                          bo, workspace, workspace_bytes);
+                          bo, workspace, workspace_bytes, sh);
 }
 
 DT_EXPORT dt_status dt_sdpa_f16_static(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D, int32_t n_qseg,
@@ -251,28 +279,19 @@ DT_EXPORT dt_status dt_sdpa_f16_static(dt_stream stream, int32_t B, int32_t Hq, 
                                        const dt_seq_segment* v_seg, const uint16_t* rot_q, const uint16_t* rot_k,
                                        float eps, dt_view4 o, float scale, const uint16_t* Wo, const uint16_t* bo) {
   using namespace dt;
-  if (B < 0 || Hq <= 0 || Hk <= 0 || D <= 0 || n_qseg <= 0 || n_kvseg <= 0 || !q_seg || !k_seg) return DT_INVALID;
-  // the scratch this request needs, by the same rule as dt_sdpa_workspace_bytes
-  int64_t Sq = 0, Skv = 0;
-  bool prep = rot_q || rot_k;
-  for (int i = 0; i < n_qseg; i++) {
-    if (q_seg[i].len < 0) return DT_INVALID;
-    Sq += q_seg[i].len;
-    prep = prep || q_seg[i].gamma;
-  }
-  for (int i = 0; i < n_kvseg; i++) {
-    if (k_seg[i].len < 0) return DT_INVALID;
-    Skv += k_seg[i].len;
-    prep = prep || k_seg[i].gamma;
-  }
-  const size_t need = dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, prep ? 1 : 0, Wo ? 1 : 0);
-  if (need > (size_t)DT_SDPA_STATIC_SCRATCH_BYTES) return DT_OOM;  // beyond the fixed array: use dt_sdpa_f16
+  // the same argument checks as dt_sdpa_f16, in the same order, before the size of the request is looked at
+  SdpaShape sh;
+  if (const dt_status st = sdpa_validate(B, Hq, Hk, D, n_qseg, q_seg, n_kvseg, k_seg, v_seg, rot_q, rot_k, o, Wo, sh);
+      st != DT_OK)
+    return st;
+  if (sh.empty) return DT_OK;
+  if (sh.need > (size_t)DT_SDPA_STATIC_SCRATCH_BYTES) return DT_OOM;  // beyond the fixed array: use dt_sdpa_f16
   void* ws = nullptr;
-  if (need > 0) {
+  if (sh.need > 0) {
     if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
     ws = sdpa_static_scratch();
     if (!ws) return DT_DEVICE_ERROR;
   }
   return sdpa_enqueue(stream, B, Hq, Hk, D, n_qseg, q_seg, n_kvseg, k_seg, v_seg, rot_q, rot_k, eps, o, scale, Wo, bo,
-                      ws, need);
+                      ws, sh.need, sh);
 }

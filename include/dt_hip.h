@@ -15,9 +15,12 @@
  *   -1  DT_INVALID     bad shape / alignment / NULL pointer / unknown qbits
  *   -2  DT_NO_KERNEL   valid request this library has no kernel for
  *   -3  DT_OOM         workspace too small
- *   -4  DT_DEVICE_ERROR the HIP runtime already held an error when the call was made (left in place for its owner;
- *                      nothing was enqueued), or the device failed under the launch; no ccv counterpart: a shim
- *                      maps it to CCV_NNC_EXEC_INVALID
+ *   -4  DT_DEVICE_ERROR the HIP runtime already reported a fault when the call was made (a faulted kernel, a lost
+ *                      device or context: left in place for its owner; nothing was enqueued), or the device failed
+ *                      under the launch; no ccv counterpart: a shim maps it to CCV_NNC_EXEC_INVALID.  A stale
+ *                      non-fatal code in the calling thread's error slot (hipErrorInvalidValue of a pointer probe,
+ *                      hipErrorPeerAccessAlreadyEnabled, hipErrorNotSupported, ...) does not refuse the call: the
+ *                      call that produced it has returned it already, and the entry point clears it
  *
  * The operator surface this replaces is the one the reference's model
  * builders call (reference paths relative to Libraries/SwiftDiffusion/Sources):

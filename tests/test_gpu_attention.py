@@ -133,7 +133,7 @@ SDPA_CASES = [
     (1, 70, 77, 8, 8, 40),        # SD1.5 cross-attention shape (D = 40, 77 keys)
     (2, 300, 300, 8, 8, 40),      # SD1.5 self-attention (reduced sequence)
     (1, 130, 190, 4, 2, 64),      # grouped heads, D = 64
-    (1, 2100, 150, 2, 1, 128),    # long query side -> 64-row-per-wave kernel, grouped heads
+    (1, 2100, 150, 2, 1, 128),    # long query side (nine 256-row workgroups per head), grouped heads
     (1, 2050, 257, 2, 2, 64),
 ]
 
@@ -287,6 +287,48 @@ def test_sdpa_rejects_bad_arguments(dthip, torch_cuda):
         dthip.sdpa_segments([z(1, 8, 2, 64)], [z(1, 0, 2, 64)], [z(1, 0, 2, 64)], 1.0)  # no keys
     assert e.value.status == dthip.DT_INVALID
     assert dthip.sdpa_segments([z(1, 0, 2, 64)], [z(1, 4, 2, 64)], [z(1, 4, 2, 64)], 1.0).shape == (1, 0, 2, 64)
+
+
+def test_entry_points_run_past_a_stale_benign_runtime_error(dthip, oracle, torch_cuda):
+    """A host that checks HIP return codes directly (as ccv does) leaves non-fatal codes in the thread's error slot:
+    a rejected argument, a second hipDeviceEnablePeerAccess.  The entry points must not take such a leftover for a
+    fault: they run, and their own launch status is what they return."""
+    import ctypes
+
+    torch = torch_cuda
+    dthip.lib()
+    hip = ctypes.CDLL("libamdhip64.so.7")  # the runtime already loaded in this process (same soname)
+    for f in (hip.hipPeekAtLastError, hip.hipGetLastError):
+        f.restype, f.argtypes = ctypes.c_int, []
+    hip.hipMemcpy.restype = ctypes.c_int
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    hip.hipDeviceEnablePeerAccess.restype = ctypes.c_int
+    hip.hipDeviceEnablePeerAccess.argtypes = [ctypes.c_int, ctypes.c_uint]
+    torch.cuda.synchronize()
+    hip.hipGetLastError()
+    rng = np.random.default_rng(77)
+    q, k, v = rand_qkv(rng, 1, 96, 80, 2, 2, 64)
+    want = oracle.C.sdpa(q, k, v, 0.125)
+    x = f16(rng.standard_normal((40, 64)))
+    w = f16(rng.standard_normal((24, 64)) * 0.1)
+    provoked = 0
+    for provoke in (lambda: hip.hipMemcpy(None, None, 16, 3), lambda: hip.hipDeviceEnablePeerAccess(0, 0)):
+        rc = provoke()
+        if rc == 0 or hip.hipPeekAtLastError() == 0:
+            continue  # this runtime does not keep that one
+        provoked += 1
+        print("stale runtime error left in place:", rc, flush=True)
+        got = dthip.sdpa_segments([to_dev(torch, q)], [to_dev(torch, k)], [to_dev(torch, v)], 0.125)
+        torch.cuda.synchronize()
+        mx, rr = oracle.err_stats(got.cpu().numpy(), want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+        assert hip.hipPeekAtLastError() == 0
+        provoke()
+        y = dthip.dense_multi(to_dev(torch, x), [dthip.QxTensor.from_f16(w)], [None])[0]
+        torch.cuda.synchronize()
+        mx, rr = oracle.err_stats(y.cpu().numpy(), oracle.C.dense(x, w, None))
+        assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+    assert provoked >= 1, "no benign runtime error could be provoked"
 
 
 def test_sdpa_flux_full_size_sampled(dthip, oracle, torch_cuda):
@@ -507,3 +549,74 @@ def test_sdpa_wan_cross_attention_full_size_sampled(dthip, oracle, torch_cuda):
     vc = torch.randn((1, 1, H, D), device="cuda", generator=gen).half().expand(B, Skv, H, D).contiguous()
     oc = dthip.ScaledDotProductAttention(scale=scale)(qd, kd, vc)
     assert float((oc.float() - vc[:, :1].float()).abs().max()) <= 2e-3
+
+
+def test_qk_row_norm_rope_wan_full_size(dthip, oracle, torch_cuda):
+    """Wan 14B at full size: RMSNorm(axis: [2]) over the 5120-wide row of all 32760 tokens, then the 3-axis rotation
+    (table 21 x 30 x 52, dims 44 / 42 / 42) and the .scale1 pre-multiplication by 128^(-1/4), in place
+    (Models/Wan.swift:87-98).  Sampled rows against the oracle, one fp16 ulp per stage."""
+    torch = torch_cuda
+    gt, gh, gw, H, D = 21, 30, 52, 40, 128
+    S, C = gt * gh * gw, H * D
+    assert S == 32760
+    g = torch.Generator(device="cuda").manual_seed(5120)
+    x = torch.randn((1, S, C), device="cuda", generator=g).half()
+    gam = f16(1 + 0.02 * np.random.default_rng(3).standard_normal(C))
+    rot = f16(dthip.WanRotaryPositionEmbedding(gh, gw, gt, channels=D))
+    assert rot.shape == (S, D)
+    rows = np.sort(np.unique(np.concatenate([[0, 1, S - 1, gh * gw - 1, gh * gw],
+                                             np.random.default_rng(4).choice(S, size=27, replace=False)])))
+    xs = x[0, torch.from_numpy(rows).cuda()].cpu().numpy()
+    post = float(128 ** -0.25)
+    print("row norm + rope at the Wan shape", flush=True)
+    y = dthip.qk_norm_rope_(x.view(1, S, H, D), to_dev(torch, gam), 1e-6, False, rot=to_dev(torch, rot),
+                            post_scale=post)
+    got = y[0, torch.from_numpy(rows).cuda()].cpu().numpy()
+    normed = oracle.C.rmsnorm(xs, gam, 1e-6).reshape(rows.size, H, D)
+    rotated = oracle.C.cmul(normed, rot[rows])
+    want = (rotated.astype(np.float32) * np.float32(post)).astype(np.float16)
+    # one ulp per stage (norm, rotation, scale), on the scale of the rotated pair's magnitude
+    pair = np.sqrt((rotated.astype(np.float64).reshape(rows.size, H, D // 2, 2) ** 2).sum(-1, keepdims=True))
+    tol = 3 * (np.broadcast_to(pair, (rows.size, H, D // 2, 2)).reshape(rows.size, H, D) * post * 2.0 ** -10 + 2.0 ** -24)
+    assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= tol)
+    # the rest of the tensor was processed too: every row has unit RMS before gamma, so no element can be large
+    assert bool(torch.isfinite(y.float()).all()) and float(y.float().abs().max()) < 40.0
+
+
+def test_sdpa_wan_causal_chunked_windows(dthip, oracle, torch_cuda):
+    """Wan causal inference (Models/Wan.swift:104-127): the frames are attended in chunks; query chunk i (rows
+    [i * frames, (i + 1) * frames)) sees the key / value prefix of min(hw, (i + 1) * frames + padFrames) rows.  Each
+    chunk is one call on offset views of the same [1, hw, h, k] tensors, its output written into its slice of one
+    buffer (the reference's Concat(axis: 1))."""
+    torch = torch_cuda
+    rng = np.random.default_rng(104)
+    time_, per_frame, H, D = 7, 90, 3, 128       # 7 latent frames of 90 tokens
+    causal, pad = 2, 1                            # chunks of 2 frames, one frame of look-ahead
+    hw = time_ * per_frame
+    frames, pad_frames = per_frame * causal, per_frame * pad
+    q, k, v = rand_qkv(rng, 1, hw, hw, H, H, D)
+    # the .scale1 convention: queries and keys pre-multiplied by 128^(-1/4), scale 1
+    q *= np.float16(128 ** -0.25)
+    k *= np.float16(128 ** -0.25)
+    scale = 1.0
+    qd, kd, vd = (to_dev(torch, t) for t in (q, k, v))
+    out = torch.full((1, hw, H, D), float("nan"), dtype=torch.float16, device="cuda")
+    n_chunks = (time_ + causal - 1) // causal
+    print("wan causal windows", n_chunks, "chunks", flush=True)
+    for i in range(n_chunks):
+        lo, hi = i * frames, min(hw, (i + 1) * frames)
+        kv = min(hw, (i + 1) * frames + pad_frames)
+        dthip.sdpa_segments([qd[:, lo:hi]], [kd[:, :kv]], [vd[:, :kv]], scale, out=out[:, lo:hi])
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.isfinite(got.astype(np.float32)).all()
+    for i in range(n_chunks):
+        lo, hi = i * frames, min(hw, (i + 1) * frames)
+        kv = min(hw, (i + 1) * frames + pad_frames)
+        want = oracle.C.sdpa(np.ascontiguousarray(q[:, lo:hi]), np.ascontiguousarray(k[:, :kv]),
+                             np.ascontiguousarray(v[:, :kv]), scale)
+        mx, rr = oracle.err_stats(got[:, lo:hi], want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (i, mx, rr)
+    # the windows matter: the first chunk's rows differ from full (non-causal) attention over all frames
+    full = oracle.C.sdpa(np.ascontiguousarray(q[:, :frames]), k, v, scale)
+    assert float(np.abs(full.astype(np.float32) - got[:, :frames].astype(np.float32)).max()) > 1e-2

@@ -802,3 +802,30 @@ def test_lora_dense_high_precision(dthip, oracle, torch_cuda, M, N, K, q, nib, r
     g = layer(xd, post=dthip.DensePost(dthip.ACT_GELU_TANH))
     o = dthip.dense_post(xd, [w], [bd], [dthip.DensePost(dthip.ACT_GELU_TANH, addend=br)])[0]
     assert torch.equal(g, o)
+
+
+@pytest.mark.parametrize("M,K,N,codec", [(8192, 320, 320, "q6p"), (8192, 320, 320, "f16"), (154, 768, 320, "q6p"),
+                                         (154, 768, 320, "f16")])
+def test_dense_sd15_shapes_full_size(dthip, oracle, M, K, N, codec):
+    """SD 1.5 attention projections at full size (Models/UNet.swift:105-107, 277-279, 307): toqueries / tokeys /
+    tovalues / unifyheads 320 -> 320 over batch 2 x 4096 tokens, and the cross-attention tokeys / tovalues
+    768 -> 320 over 2 x 77 context tokens; palettized (q6p) and plain fp16 weights, every output element."""
+    import torch
+
+    rng = np.random.default_rng(M + K)
+    x = (rng.standard_normal((M, K))).astype(np.float16)
+    b = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    if codec == "f16":
+        w = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+        qx = dthip.QxTensor.from_f16(w)
+        want = oracle.C.dense(x, w, b)
+    else:
+        q, nib = dthip.CODEC[codec]
+        packed, _, _ = oracle.synth_qx_weight(rng, N, K, q, nib, 0.05)
+        qx = dthip.QxTensor.from_packed(packed, q, nib, (N, K))
+        want = oracle.C.dense_qx(x, packed, q, nib, N, b)
+    print("dense sd1.5 shape", M, K, N, codec, flush=True)
+    got = dthip.dense_multi(dev(x), [qx], [dev(b)])[0].cpu().numpy()
+    mx, rr = oracle.err_stats(got, want)
+    assert mx <= 2e-2 and rr <= 1e-3, (mx, rr)

@@ -217,3 +217,105 @@ def test_unet_transformer_block_vs_oracle(dthip, oracle, k, h, b, gs, t, cw, q):
     print("x max-abs", mx, "rel-rms", rr, "scale", float(np.abs(want.astype(np.float32)).max()), flush=True)
     assert mx <= 2e-2 and rr <= 2e-3
 
+
+
+def test_flux_step_full_size_sampled(dthip, oracle):
+    """The benchmark's own step at full size -- 512 text + 4096 image tokens, 24 heads x 128, q6p (nib 4096) -- as
+    the exact three calls the benchmark makes: the grouped QKV launch (image and context problems, per-head RMSNorm
+    + RoPE in the epilogue, rot_pos0 512 / 0) writing one strided [S, 3, H, D] buffer; attention reading Q, K, V as
+    strided views of that buffer; the grouped output projections.  Sampled token rows (0, 511, 512 and 4607 among
+    them) against the oracle's op-by-op chain Dense -> RMSNorm -> cmul -> attention -> Dense
+    (Models/Flux1.swift:161-245) at the block bar."""
+    import torch
+
+    T, gh, gw, H, D, q, nib = 512, 64, 64, 24, 128, 6, 4096
+    HW, C = gh * gw, H * D
+    S = T + HW
+    rng = np.random.default_rng(4608)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    f16 = lambda a: np.asarray(a, dtype=np.float16)
+    packs, w, bias = {}, {}, {}
+    for name in ("c_q", "c_k", "c_v", "x_q", "x_k", "x_v", "c_o", "x_o"):
+        packs[name], _, _ = oracle.synth_qx_weight(rng, C, C, q, nib)
+        w[name] = dthip.QxTensor.from_packed(packs[name], q, nib, (C, C))
+        bias[name] = f16(rng.standard_normal(C) * 0.02)
+    gam = {n: f16(1 + 0.02 * rng.standard_normal(D)) for n in ("c_q", "c_k", "x_q", "x_k")}
+    rot = f16(dthip.Flux1RotaryPositionEmbedding(gh, gw, T, channels=D))
+    ctx, img = f16(rng.standard_normal((T, C))), f16(rng.standard_normal((HW, C)))
+    scale = 1.0 / float(np.sqrt(D))
+
+    # ---- the benchmark's three calls
+    qkv = torch.full((S, 3, H, D), float("nan"), dtype=torch.float16, device="cuda")
+    att = torch.full((1, S, H, D), float("nan"), dtype=torch.float16, device="cuda")
+    out_c = torch.full((T, C), float("nan"), dtype=torch.float16, device="cuda")
+    out_x = torch.full((HW, C), float("nan"), dtype=torch.float16, device="cuda")
+    qkv2 = qkv.view(S, 3 * C)
+    views = lambda lo, hi: [qkv2[lo:hi, i * C:(i + 1) * C] for i in range(3)]
+    d_rot = dev(rot)
+    epi = lambda s, pos0: [dthip.HeadEpilogue(dev(gam[s + "_q"]), d_rot, pos0, 1e-6, D),
+                           dthip.HeadEpilogue(dev(gam[s + "_k"]), d_rot, pos0, 1e-6, D), None]
+    d_ctx, d_img = dev(ctx), dev(img)
+    d_bias = {n: dev(b) for n, b in bias.items()}
+    print("flux step at full size: grouped QKV", flush=True)
+    dthip.dense_grouped([
+        dict(x=d_img, weights=[w["x_q"], w["x_k"], w["x_v"]], biases=[d_bias["x_q"], d_bias["x_k"], d_bias["x_v"]],
+             outs=views(T, S), epilogues=epi("x", T)),
+        dict(x=d_ctx, weights=[w["c_q"], w["c_k"], w["c_v"]], biases=[d_bias["c_q"], d_bias["c_k"], d_bias["c_v"]],
+             outs=views(0, T), epilogues=epi("c", 0))])
+    print("flux step at full size: attention on strided views", flush=True)
+    q4, k4, v4 = (qkv[:, i].unsqueeze(0) for i in range(3))
+    dthip.sdpa_segments([q4], [k4], [v4], scale, out=att)
+    print("flux step at full size: grouped out-projections", flush=True)
+    att2 = att.view(S, C)
+    dthip.dense_grouped([dict(x=att2[T:], weights=[w["x_o"]], biases=[d_bias["x_o"]], outs=[out_x]),
+                         dict(x=att2[:T], weights=[w["c_o"]], biases=[d_bias["c_o"]], outs=[out_c])])
+    torch.cuda.synchronize()
+    got_qkv, got_att = qkv.cpu().numpy(), att.cpu().numpy()[0]
+    got_out = np.concatenate([out_c.cpu().numpy(), out_x.cpu().numpy()])
+    assert np.isfinite(got_qkv.astype(np.float32)).all() and np.isfinite(got_out.astype(np.float32)).all()
+
+    # ---- the oracle: K and V for every token, Q / attention / output for the sampled rows
+    rows = np.sort(np.unique(np.concatenate([[0, 255, 256, T - 1, T, T + 255, T + 256, S - 257, S - 256, S - 1],
+                                             rng.choice(S, size=14, replace=False)])))
+    x_all = np.concatenate([ctx, img])
+    heads = lambda a: a.reshape(-1, H, D)
+
+    def proj(n, sel=None):
+        """Dense of stream-specific weights over the joint sequence's rows (all, or the selected ones)."""
+        idx = np.arange(S) if sel is None else sel
+        out = np.empty((idx.size, C), dtype=np.float16)
+        for s, lo, hi in (("c", 0, T), ("x", T, S)):
+            m = (idx >= lo) & (idx < hi)
+            if m.any():
+                out[m] = oracle.C.dense_qx(np.ascontiguousarray(x_all[idx[m]]), packs[f"{s}_{n}"], q, nib, C, bias[f"{s}_{n}"])
+        return out
+
+    def norm_rot(y, n, idx):
+        out = np.empty((idx.size, H, D), dtype=np.float16)
+        for s, lo, hi in (("c", 0, T), ("x", T, S)):
+            m = (idx >= lo) & (idx < hi)
+            if m.any():
+                out[m] = oracle.C.cmul(oracle.C.rmsnorm(heads(y[m]), gam[f"{s}_{n}"], 1e-6), rot[idx[m]])
+        return out
+
+    all_rows = np.arange(S)
+    want_k = norm_rot(proj("k"), "k", all_rows)
+    want_v = heads(proj("v"))
+    want_q = norm_rot(proj("q", rows), "q", rows)
+    # the projections with their fused epilogue, where they landed in the strided buffer
+    for name, g, wnt in (("q", got_qkv[rows, 0], want_q), ("k", got_qkv[:, 1], want_k), ("v", got_qkv[:, 2], want_v)):
+        mx, rr = oracle.err_stats(g, wnt)
+        print("qkv", name, "max-abs", mx, "rel-rms", rr, flush=True)
+        assert mx <= 2e-2 and rr <= 1e-3, (name, mx, rr)
+    want_att = oracle.C.sdpa(want_q[None], want_k[None], want_v[None], scale)[0]
+    mx, rr = oracle.err_stats(got_att[rows], want_att)
+    print("attention max-abs", mx, "rel-rms", rr, flush=True)
+    assert mx <= 2e-2 and rr <= 1e-3, (mx, rr)
+    want_out = np.empty((rows.size, C), dtype=np.float16)
+    for s, lo, hi in (("c", 0, T), ("x", T, S)):
+        m = (rows >= lo) & (rows < hi)
+        want_out[m] = oracle.C.dense_qx(np.ascontiguousarray(want_att[m].reshape(-1, C)), packs[f"{s}_o"], q, nib, C,
+                                        bias[f"{s}_o"])
+    mx, rr = oracle.err_stats(got_out[rows], want_out)
+    print("out max-abs", mx, "rel-rms", rr, flush=True)
+    assert mx <= 2e-2 and rr <= 2e-3, (mx, rr)

@@ -55,12 +55,16 @@ def test_static_scratch_entry_point_matches_workspace_entry_point(dthip, oracle,
     cases = [_case(dthip, oracle, torch, rng, *sz, fused_out) for sz in sizes]
     outs = [torch.full(shape, float("nan"), dtype=torch.float16, device="cuda") for _, _, shape in cases]
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # torch's own count sees its caching allocator only; the driver's free-byte count sees any hipMalloc / hipFree
+    # that the library itself might make
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     for (args, _, _), out in zip(cases, outs):
         print("static scratch call", tuple(out.shape), "fused_out" if fused_out else "fused_prep", flush=True)
         dthip.sdpa_segments(**args, out=out, static_scratch=True)
     assert torch.cuda.memory_allocated() == before  # the host mirror allocated nothing either
+    assert torch.cuda.mem_get_info()[0] == free_before  # nor did the library, behind torch's back
     torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
     for (args, want, _), out in zip(cases, outs):
         ref = dthip.sdpa_segments(**args)  # the existing entry point, workspace allocated by the caller
         assert torch.equal(out, ref)
@@ -82,3 +86,52 @@ def test_static_scratch_rejects_requests_beyond_the_array(dthip):
     # without staging the same shapes need no scratch at all and run
     o = dthip.sdpa_segments([q[:, :256]], [q[:, :256]], [q[:, :256]], 1.0, static_scratch=True)
     assert o.shape == (B, 256, H, D)
+
+
+def test_static_scratch_at_the_documented_flux_shape(dthip):
+    """The shape the array is sized for: 512 text + 64 x 64 image tokens, 24 heads x 128, fused per-head RMSNorm and
+    RoPE (staged Q and K: 56.6 MB, reaching the far end of the 64 MiB array) -- bit for bit against dt_sdpa_f16."""
+    import torch
+
+    T, h, w, H, D = 512, 64, 64, 24, 128
+    HW = h * w
+    assert dthip.lib().dt_sdpa_workspace_bytes(1, H, H, D, T + HW, T + HW, 1, 0) <= dthip.STATIC_SCRATCH_BYTES
+    g = torch.Generator(device="cuda").manual_seed(72)
+    rnd = lambda *s: torch.randn(s, device="cuda", generator=g).half()
+    segs = {n: (rnd(1, T, H, D), rnd(1, HW, H, D)) for n in "qkv"}
+    gam = {n: ((1 + 0.05 * rnd(D).float()).half(), (1 + 0.05 * rnd(D).float()).half()) for n in "qk"}
+    rot = torch.from_numpy(dthip.Flux1RotaryPositionEmbedding(h, w, T, channels=D).astype(np.float16)).cuda()
+    args = dict(q_segs=list(segs["q"]), k_segs=list(segs["k"]), v_segs=list(segs["v"]), scale=1 / np.sqrt(D),
+                gamma_q=list(gam["q"]), gamma_k=list(gam["k"]), rot_q=rot, rot_k=rot)
+    out = torch.full((1, T + HW, H, D), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    print("static scratch call at the Flux shape", tuple(out.shape), flush=True)
+    dthip.sdpa_segments(**args, out=out, static_scratch=True)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    ref = dthip.sdpa_segments(**args)
+    assert torch.equal(out, ref)
+    assert bool(torch.isfinite(out.float()).all())
+
+
+def test_static_scratch_validates_like_the_workspace_entry_point(dthip):
+    """Bad arguments get the status dt_sdpa_f16 gives them, also when the shapes are beyond the array: the size of
+    the request is looked at only after the argument checks."""
+    import torch
+
+    z = lambda *s: torch.zeros(s, dtype=torch.float16, device="cuda")
+    g = torch.ones(128, dtype=torch.float16, device="cuda")
+    big = 9000  # staged Q + K beyond 64 MiB at 24 heads x 128
+    cases = [
+        (dict(q_segs=[z(1, big, 24, 128)], k_segs=[z(1, big, 5, 128)], v_segs=[z(1, big, 5, 128)]), dthip.DT_INVALID),  # 5 does not divide 24
+        (dict(q_segs=[z(1, big, 24, 136)], k_segs=[z(1, big, 24, 136)], v_segs=[z(1, big, 24, 136)]), dthip.DT_NO_KERNEL),  # D > 128
+        (dict(q_segs=[z(1, big, 24, 128)], k_segs=[z(1, big, 24, 128)], v_segs=[z(1, big - 8, 24, 128)]), dthip.DT_INVALID),  # k / v lengths differ
+        (dict(q_segs=[z(1, 8, 2, 64)], k_segs=[z(1, 0, 2, 64)], v_segs=[z(1, 0, 2, 64)]), dthip.DT_INVALID),  # no keys
+    ]
+    for kw, want in cases:
+        for static in (False, True):
+            with pytest.raises(dthip.DtError) as e:
+                gq = [g[:kw["q_segs"][0].shape[-1]]] if kw["q_segs"][0].shape[-1] <= 128 else None
+                dthip.sdpa_segments(**kw, scale=1.0, gamma_q=gq, static_scratch=static)
+            assert e.value.status == want, (static, want, e.value.status)
