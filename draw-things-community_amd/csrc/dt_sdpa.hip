@@ -17,6 +17,9 @@
 // the V^T operand (head dimension along lanes, keys along registers) comes
 // from ds_read_b64_tr_b16, which hands lane j of a 16-lane group the element
 // column (j % 4) of the rows addressed by lanes (j / 4) + {0, 4, 8, 12}.
+#include <atomic>
+#include <cstdlib>
+
 #include "dt_common.h"
 #include "dt_sdpa.h"
 
@@ -49,7 +52,15 @@ __device__ __forceinline__ int v_unit_swz(int row, int u) {
   return u ^ ((row >> 1) & 1);
 }
 
-template <int DP, bool PREMUL, bool ONESEG>
+// SPLIT: the (task, key tile) pairs of the whole launch -- a task being the 256 query rows of one (batch, head) --
+// are laid end to end and cut into one equal run per workgroup, so that a launch whose task count is no multiple
+// of the compute units still keeps all of them busy to the end.  A workgroup walks its run task by task.  A piece
+// that covers a whole task is finished as usual.  Any other piece leaves its unnormalised fp32 output, reference
+// maximum and row sums in a workspace slot and adds its tile count to the task's counter; the piece that brings the
+// counter to the task's tile count -- the last to arrive, whichever that is -- folds all the task's pieces together,
+// in the fixed order of their workgroups, and writes the output.  Nobody waits for anybody: there is no spinning
+// anywhere, and the result does not depend on which piece arrives last.
+template <int DP, bool PREMUL, bool ONESEG, bool SPLIT>
 __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   constexpr int ROWB = DP * 2;                 // bytes per tile row
   constexpr int DCH = DP / 8;                  // 16-byte chunks per row
@@ -79,13 +90,78 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     const int per = a.total_blocks / 8;
     if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
   }
-  const int qt = bid % a.q_tiles;
-  const int bh = bid / a.q_tiles;
+  const int64_t Sq = a.Sq, Skv = a.Skv;
+  const int D = a.D;
+  const int n_tiles = (int)((Skv + BKV - 1) / BKV);
+
+  // ---- per-thread constants of the K / V tile loaders ---------------------
+  // Tiles go from memory straight into LDS.  A wave's transfer instruction
+  // fills 1 KB of a tile, lane l landing on its 16-byte slot l; each thread
+  // issues LOADS of them per K tile and per V tile and fetches the chunk that
+  // the swizzle assigns to its slot.  Lanes whose row lies past the last key,
+  // or whose chunk lies past D, stay idle: those slots keep what they held
+  // (zeros from the start, or an earlier tile's finite values), which the
+  // masked scores and the zero padding of Q make harmless.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  int ld_row[LOADS], k_ch[LOADS], v_ch[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; i++) {
+    const int off = (wave * LOADS + i) * 1024 + lane * 16;
+    const int row = off / ROWB, pc = (off % ROWB) / 16;
+    ld_row[i] = row;
+    k_ch[i] = k_chunk_swz<DP>(row, pc);  // the swizzles are involutions
+    v_ch[i] = v_unit_swz<DP>(row, pc >> 2) * 4 + (pc & 3);
+  }
+  // slots that no transfer will ever write must not hold NaN patterns
+  if (D < DP || Skv % BKV != 0) {
+    for (int i = tid * 16; i < TILE_B; i += 512 * 16) {
+      *reinterpret_cast<uint4_t*>(Ks0 + i) = uint4_t{0, 0, 0, 0};
+      *reinterpret_cast<uint4_t*>(Ks1 + i) = uint4_t{0, 0, 0, 0};
+      *reinterpret_cast<uint4_t*>(Vs0 + i) = uint4_t{0, 0, 0, 0};
+      *reinterpret_cast<uint4_t*>(Vs1 + i) = uint4_t{0, 0, 0, 0};
+    }
+    __syncthreads();
+  }
+
+  // ---- per-lane LDS read offsets --------------------------------------------
+  // K operand: key row kb*32 + l32, chunk 2*ks + hi
+  int k_rd[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) k_rd[ks] = l32 * ROWB + k_chunk_swz<DP>(l32, 2 * ks + hi) * 16;
+  // V^T operand through the transposing read: lane i of a 16-lane group addresses
+  // key row (i / 4) of a 4-key run and 4 head-dim elements at 4 * (i % 4); the
+  // two groups of a half-wave cover head-dim 0..15 and 16..31 of block db.
+  const int li = lane & 15, dg = (lane >> 4) & 1;
+  int v_rd[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++) {
+    const int row = 4 * hi + (li >> 2);  // + multiples of 4 per k-step: the swizzle depends on row & 3 (or (row >> 1) & 1) only
+    v_rd[db] = row * ROWB + v_unit_swz<DP>(row, db) * 64 + dg * 32 + (li & 3) * 8;
+  }
+  const float c = PREMUL ? 1.0f : a.scale_log2e;
+
+  // ---- the run of work of this workgroup ----------------------------------
+  // Not SPLIT: one task, all of its key tiles.  SPLIT: units [u, u_end) of the launch's (task, key tile) pairs.
+  int u = 0, u_end = 0;  // (a split launch holds fewer than 2^31 units)
+  if constexpr (SPLIT) {
+    u = (int)((int64_t)bid * a.units / a.total_blocks);
+    u_end = (int)((int64_t)(bid + 1) * a.units / a.total_blocks);
+  }
+  [[maybe_unused]] int piece_no = 0;
+  [[maybe_unused]] __shared__ int s_last;
+  for (;;) {
+  int task = bid, t_lo = 0, t_hi = n_tiles;
+  if constexpr (SPLIT) {
+    if (u >= u_end) break;
+    task = u / n_tiles;
+    t_lo = u - task * n_tiles;
+    t_hi = (u_end - u) < (n_tiles - t_lo) ? t_lo + (u_end - u) : n_tiles;
+  }
+  const int qt = task % a.q_tiles;
+  const int bh = task / a.q_tiles;
   const int h = bh % a.Hq;
   const int b = bh / a.Hq;
   const int hk = h / a.group;
-  const int64_t Sq = a.Sq, Skv = a.Skv;
-  const int D = a.D;
 
   // ---- Q^T fragments straight from global memory -----------------------
   // B operand of K Q^T: lane holds query column l32, head-dim slots 16*ks + 8*hi + 0..7.
@@ -108,23 +184,6 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   }
 
   // ---- K / V tile loaders ------------------------------------------------
-  // Tiles go from memory straight into LDS.  A wave's transfer instruction
-  // fills 1 KB of a tile, lane l landing on its 16-byte slot l; each thread
-  // issues LOADS of them per K tile and per V tile and fetches the chunk that
-  // the swizzle assigns to its slot.  Lanes whose row lies past the last key,
-  // or whose chunk lies past D, stay idle: those slots keep what they held
-  // (zeros from the start, or an earlier tile's finite values), which the
-  // masked scores and the zero padding of Q make harmless.
-  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  int ld_row[LOADS], k_ch[LOADS], v_ch[LOADS];
-#pragma unroll
-  for (int i = 0; i < LOADS; i++) {
-    const int off = (wave * LOADS + i) * 1024 + lane * 16;
-    const int row = off / ROWB, pc = (off % ROWB) / 16;
-    ld_row[i] = row;
-    k_ch[i] = k_chunk_swz<DP>(row, pc);  // the swizzles are involutions
-    v_ch[i] = v_unit_swz<DP>(row, pc >> 2) * 4 + (pc & 3);
-  }
   // ONESEG: K and V are one run of rows each and small enough for 32-bit byte
   // offsets from a uniform base; a tile step adds a uniform stride.
   // Otherwise the segment of a tile is looked up once per tile (uniformly): a
@@ -134,7 +193,8 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   const char* k_base = nullptr;
   const char* v_base = nullptr;
   uint32_t k_step = 0, v_step = 0;
-  int rows_left = (int)(Skv < 0x7fffffff ? Skv : 0x7fffffff);  // ONESEG: keys from the next K tile on
+  const int64_t keys_ahead = Skv - (int64_t)t_lo * BKV;                     // keys from this piece's first tile on
+  int rows_left = (int)(keys_ahead < 0x7fffffff ? keys_ahead : 0x7fffffff);  // ONESEG: keys from the next K tile on
   int rows_left_v = rows_left;
   if constexpr (ONESEG) {
     k_base = reinterpret_cast<const char*>(a.k[0].ptr + b * a.k[0].sb + hk * a.k[0].sh);
@@ -143,8 +203,8 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     v_step = (uint32_t)(a.v[0].ss * BKV * 2);
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
-      k_off[i] = (uint32_t)((ld_row[i] * a.k[0].ss + k_ch[i] * 8) * 2);
-      v_off[i] = (uint32_t)((ld_row[i] * a.v[0].ss + v_ch[i] * 8) * 2);
+      k_off[i] = (uint32_t)((ld_row[i] * a.k[0].ss + k_ch[i] * 8) * 2) + (uint32_t)t_lo * k_step;
+      v_off[i] = (uint32_t)((ld_row[i] * a.v[0].ss + v_ch[i] * 8) * 2) + (uint32_t)t_lo * v_step;
     }
   }
   // General case: a uniform cursor holds the segment the next tile starts in --
@@ -158,7 +218,8 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     int64_t end;       // first joint row past the segment
     int64_t row0;      // first joint row of the next tile
   };
-  SegCursor kcur{nullptr, 0, 0, 0}, vcur{nullptr, 0, 0, 0};
+  // (an end of 0 makes the first tile look its segment up)
+  SegCursor kcur{nullptr, 0, 0, (int64_t)t_lo * BKV}, vcur{nullptr, 0, 0, (int64_t)t_lo * BKV};
   auto seek = [&](const SdpaSeg* segs, SegCursor& c, uint32_t (&off)[LOADS], const int (&chs)[LOADS])
                   __attribute__((always_inline)) {
     int sg = 0;
@@ -230,33 +291,6 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       issue_general(a.v, vcur, v_off, v_ch, dst);
     }
   };
-  // slots that no transfer will ever write must not hold NaN patterns
-  if (D < DP || Skv % BKV != 0) {
-    for (int i = tid * 16; i < TILE_B; i += 512 * 16) {
-      *reinterpret_cast<uint4_t*>(Ks0 + i) = uint4_t{0, 0, 0, 0};
-      *reinterpret_cast<uint4_t*>(Ks1 + i) = uint4_t{0, 0, 0, 0};
-      *reinterpret_cast<uint4_t*>(Vs0 + i) = uint4_t{0, 0, 0, 0};
-      *reinterpret_cast<uint4_t*>(Vs1 + i) = uint4_t{0, 0, 0, 0};
-    }
-    __syncthreads();
-  }
-
-  // ---- per-lane LDS read offsets --------------------------------------------
-  // K operand: key row kb*32 + l32, chunk 2*ks + hi
-  int k_rd[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ks++) k_rd[ks] = l32 * ROWB + k_chunk_swz<DP>(l32, 2 * ks + hi) * 16;
-  // V^T operand through the transposing read: lane i of a 16-lane group addresses
-  // key row (i / 4) of a 4-key run and 4 head-dim elements at 4 * (i % 4); the
-  // two groups of a half-wave cover head-dim 0..15 and 16..31 of block db.
-  const int li = lane & 15, dg = (lane >> 4) & 1;
-  int v_rd[DB];
-#pragma unroll
-  for (int db = 0; db < DB; db++) {
-    const int row = 4 * hi + (li >> 2);  // + multiples of 4 per k-step: the swizzle depends on row & 3 (or (row >> 1) & 1) only
-    v_rd[db] = row * ROWB + v_unit_swz<DP>(row, db) * 64 + dg * 32 + (li & 3) * 8;
-  }
-
   // ---- running state -----------------------------------------------------
   float16_t oacc[DB];
 #pragma unroll
@@ -265,9 +299,6 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     for (int v = 0; v < 16; v++) oacc[db][v] = 0.f;
   float m_ref = -INFINITY;  // reference for the exponentials (raw score units); trails the true running maximum
   float l_run = 0.f;        // this lane's share of the row sum
-
-  const float c = PREMUL ? 1.0f : a.scale_log2e;
-  const int n_tiles = (int)((Skv + BKV - 1) / BKV);
 
   float16_t sacc[2];   // S^T of the tile in flight (keys x queries)
   half8_t pf[2][2];    // its probabilities, as the B operand of the second MFMA
@@ -406,44 +437,46 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the tile has landed
   __syncthreads();
 
-  // interval t: K(t) is in k_cur, V(t-1) in v_prev; K(t+1) goes to k_next, V(t) to v_cur
+  // interval t (key tiles t_lo .. t_hi - 1 of the task): K(t) is in k_cur, V(t-1) in v_prev; K(t+1) goes to
+  // k_next, V(t) to v_cur
   auto interval = [&](int t, const unsigned char* k_cur, unsigned char* k_next, const unsigned char* v_prev,
                       unsigned char* v_cur) __attribute__((always_inline)) {
-    if (t + 1 < n_tiles) issue_k(k_next);
-    if (t < n_tiles) issue_v(v_cur);
+    if (t + 1 < t_hi) issue_k(k_next);
+    if (t < t_hi) issue_v(v_cur);
     // the wave doing softmax arithmetic gets issue priority: its exponentials only make progress in
     // the gaps the other wave's MFMA stream leaves (measured: +1 %; the opposite assignment -2 %)
     if (!second) {
       __builtin_amdgcn_s_setprio(0);
-      if (t > 0) pv_phase(v_prev);
-      if (t < n_tiles) {
+      if (t > t_lo) pv_phase(v_prev);
+      if (t < t_hi) {
         s_phase(k_cur);
         __builtin_amdgcn_s_setprio(2);
         softmax_phase(t);
       }
     } else {
-      if (t > 0) {
+      if (t > t_lo) {
         __builtin_amdgcn_s_setprio(2);
         softmax_phase(t - 1);
         __builtin_amdgcn_s_setprio(0);
         pv_phase(v_prev);
       }
-      if (t < n_tiles) s_phase(k_cur);
+      if (t < t_hi) s_phase(k_cur);
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
   };
-  for (int t = 0; t <= n_tiles; t += 2) {
+  for (int t = t_lo; t <= t_hi; t += 2) {
     interval(t, Ks0, Ks1, Vs1, Vs0);
-    if (t + 1 <= n_tiles) interval(t + 1, Ks1, Ks0, Vs0, Vs1);
+    if (t + 1 <= t_hi) interval(t + 1, Ks1, Ks0, Vs0, Vs1);
   }
+  __builtin_amdgcn_s_setprio(0);
 
   // ---- normalise and store O ----------------------------------------------
   // O^T block db: lane holds query column l32 and head-dim 8*g + 4*hi + (0..3);
   // swapping the odd groups of the low half-wave with the even groups of the
   // high half-wave leaves every lane with runs of 8 consecutive head-dim
   // elements (16-byte stores).
-  {
+  auto store_output = [&]() __attribute__((always_inline)) {
     const int64_t qi = (int64_t)qt * QROWS + wave * 32 + l32;
     const float l_tot = sum32(l_run);
     const float inv = 1.0f / l_tot;
@@ -479,7 +512,155 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
         }
       }
     }
+  };
+
+  if constexpr (!SPLIT) {
+    store_output();
+    break;
+  } else {
+    if (t_lo == 0 && t_hi == n_tiles) {
+      store_output();  // the piece is the whole task
+    } else {
+      // ---- a piece of a task: leave it for, or fold in, the task's other pieces ----------------------------
+      // Slot layout (floats): [DB * 16 accumulators][512 threads], then [512] reference maxima, then [512]
+      // row-sum shares: a wave's access covers 256 consecutive bytes.  A workgroup owns two slots: its first piece
+      // goes to the even one, a later piece -- which can only be its last -- to the odd one.
+      // The pieces of a task run on any compute units of the device, whose L2 caches (one per die) do not see each
+      // other's ordinary stores.  Partial results are therefore written and read with device-scope accesses
+      // (relaxed atomics: write-through stores, loads that do not trust a die's cached copy) instead of
+      // bracketing ordinary accesses with cache-wide write-backs and invalidations, which cost far more than the
+      // 130 KB they would protect.
+      constexpr int SLOT_F = sdpa_split_slot_floats(DP);
+      const int P = a.total_blocks;
+      float* slot = a.partials + (size_t)(2 * bid + (piece_no > 0 ? 1 : 0)) * SLOT_F;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++)
+          __hip_atomic_store(slot + (db * 16 + v) * 512 + tid, oacc[db][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(slot + DB * 16 * 512 + tid, m_ref, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(slot + DB * 16 * 512 + 512 + tid, l_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // every wave's stores have been acknowledged before the barrier, hence before the one thread's count that
+      // publishes the piece
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      __syncthreads();
+      if (tid == 0) {
+        const int done = t_hi - t_lo;
+        const int before = __hip_atomic_fetch_add(a.counters + task, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (before + done == n_tiles) ? 1 : 0;
+      }
+      __syncthreads();
+      if (s_last != 0) {  // uniform: every other piece of the task has been published
+        const int64_t ua = (int64_t)task * n_tiles, ub = ua + n_tiles;
+        // the workgroup whose run holds unit x is the largest p with p * units < (x + 1) * P
+        const int p_lo = (int)(((ua + 1) * P - 1) / a.units), p_hi = (int)((ub * P - 1) / a.units);
+        // The pieces are folded in the order of their workgroups, this one's own included (re-read from its slot),
+        // whichever of them happens to be the one doing it: the result does not depend on the order of arrival.
+        for (int p = p_lo; p <= p_hi; p++) {
+          const int64_t first_unit = (int64_t)p * a.units / P;
+          const float* other = a.partials + (size_t)(2 * p + (first_unit < ua ? 1 : 0)) * SLOT_F;
+          auto ld = [&](int i) __attribute__((always_inline)) {
+            return __hip_atomic_load(other + i * 512 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          };
+          // all of the slot's loads go out before the first of them is waited for
+          const float m_o = ld(DB * 16), l_o = ld(DB * 16 + 1);
+          float16_t got[DB];
+#pragma unroll
+          for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) got[db][v] = ld(db * 16 + v);
+          __builtin_amdgcn_sched_barrier(0);
+          if (p == p_lo) {
+            m_ref = m_o;
+            l_run = l_o;
+#pragma unroll
+            for (int db = 0; db < DB; db++) oacc[db] = got[db];
+            continue;
+          }
+          const float m_new = fmaxf(m_ref, m_o);
+          const float wa = fast_exp2((m_ref - m_new) * c), wb = fast_exp2((m_o - m_new) * c);
+          m_ref = m_new;
+          l_run = l_run * wa + l_o * wb;
+#pragma unroll
+          for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) oacc[db][v] = oacc[db][v] * wa + got[db][v] * wb;
+        }
+        store_output();
+      }
+    }
+    u += t_hi - t_lo;
+    piece_no++;
   }
+  }  // the workgroup's run
+}
+
+// Zeroes the per-task tile counters of a SPLIT launch (a fill kernel, so that the launch can be captured in a graph).
+__global__ void sdpa_zero_counters_kernel(int32_t* counters, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0;
+}
+
+// Compute units of the calling thread's current device (cached per ordinal; 256 if the runtime cannot say).
+static int compute_units() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  if (dev < 0 || dev >= 64) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+      (void)hipGetLastError();
+      n = 256;
+    }
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+bool sdpa_split_plan(int32_t B, int32_t Hq, int32_t D, int64_t Sq, int64_t Skv, SdpaSplit* plan) {
+  if (B <= 0 || Hq <= 0 || D <= 0 || Sq <= 0 || Skv <= 0) return false;
+  // DT_SDPA_KEY_SPLIT = "never" | "always" (whenever the launch can be cut at all; for tests and measurements);
+  // anything else, or unset: decide by the estimate below.  Read at every call.
+  const char* knob = getenv("DT_SDPA_KEY_SPLIT");
+  const bool never = knob && knob[0] == 'n', always = knob && knob[0] == 'a';
+  if (never) return false;
+  const int64_t tasks = (int64_t)B * Hq * ((Sq + QROWS - 1) / QROWS);
+  const int64_t n_tiles = (Skv + BKV - 1) / BKV;
+  const int64_t units = tasks * n_tiles;
+  if (tasks > (1 << 20) || units >= (1LL << 31)) return false;  // (the kernel counts units in 32 bits)
+  const int cus = compute_units();
+  // at most 8 pieces per task (the piece that arrives last folds the others in one after the other), at least
+  // `min_tiles` key tiles per workgroup
+  const int64_t min_tiles = always ? 2 : 8;
+  int64_t wgs = cus;
+  if (wgs > tasks * 8) wgs = tasks * 8;
+  if (wgs > units / min_tiles) wgs = units / min_tiles;
+  if (wgs < 2 || n_tiles < 2) return false;
+  if (!always) {
+    // Measured on this part (head size 128): the card delivers about the same attention throughput whether all of
+    // its compute units are busy or only 70-85 % of them -- a compute unit runs a key tile in ~1.4 us when a third
+    // of the card idles and in ~1.9 us when none does -- so a launch of 1.69 or 6.19 rounds of workgroups gains
+    // nothing from being cut into equal runs (0.276 against 0.248 ms at 24 heads x 4608 tokens).  What does gain
+    // is a launch that fills well under one round: there the unsplit time is one task at the fast rate, the split
+    // time the mean load at the slow rate plus ~25 us of fixed cost per workgroup (counter reset, pipeline refill,
+    // partial results out and in).
+    const double rounds = (double)tasks / cus;
+    if (rounds >= 1.0) return false;
+    const double fixed = 25.0 / (1.9 * (double)n_tiles);  // in task times
+    if (1.0 / 1.35 <= rounds * (double)cus / (double)wgs + fixed) return false;
+  }
+  if (plan) {
+    plan->workgroups = (int32_t)wgs;
+    plan->tasks = (int32_t)tasks;
+    plan->units = units;
+    plan->counter_bytes = ((size_t)tasks * 4 + 255) & ~(size_t)255;
+    plan->partial_bytes = (size_t)2 * wgs * sdpa_split_slot_floats(D <= 64 ? 64 : 128) * 4;
+  }
+  return true;
 }
 
 template <int DP>
@@ -492,13 +673,30 @@ static dt_status launch(hipStream_t s, SdpaArgs a) {
   // one K and one V segment whose rows lie within 2 GiB of the head's first row: 32-bit offsets
   const bool oneseg = a.n_kvseg == 1 && a.k[0].ss > 0 && a.v[0].ss > 0 && a.Skv < (1 << 30) &&
                       (a.Skv + 2 * BKV) * a.k[0].ss * 2 < 0x7fffffffLL && (a.Skv + 2 * BKV) * a.v[0].ss * 2 < 0x7fffffffLL;
-  dim3 grid((unsigned)total), block(512);
+  dim3 block(512);
+  if (a.partials) {
+    // key-split launch: the counters start at zero, then one workgroup per equal run of units
+    hipLaunchKernelGGL(sdpa_zero_counters_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a.counters,
+                       (int)total);
+    if (const dt_status st = launch_status(); st != DT_OK) return st;
+    a.total_blocks = a.split_workgroups;
+    dim3 grid((unsigned)a.split_workgroups);
+    if (oneseg) {
+      if (premul) hipLaunchKernelGGL((sdpa_kernel<DP, true, true, true>), grid, block, 0, s, a);
+      else hipLaunchKernelGGL((sdpa_kernel<DP, false, true, true>), grid, block, 0, s, a);
+    } else {
+      if (premul) hipLaunchKernelGGL((sdpa_kernel<DP, true, false, true>), grid, block, 0, s, a);
+      else hipLaunchKernelGGL((sdpa_kernel<DP, false, false, true>), grid, block, 0, s, a);
+    }
+    return launch_status();
+  }
+  dim3 grid((unsigned)total);
   if (oneseg) {
-    if (premul) hipLaunchKernelGGL((sdpa_kernel<DP, true, true>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((sdpa_kernel<DP, false, true>), grid, block, 0, s, a);
+    if (premul) hipLaunchKernelGGL((sdpa_kernel<DP, true, true, false>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((sdpa_kernel<DP, false, true, false>), grid, block, 0, s, a);
   } else {
-    if (premul) hipLaunchKernelGGL((sdpa_kernel<DP, true, false>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((sdpa_kernel<DP, false, false>), grid, block, 0, s, a);
+    if (premul) hipLaunchKernelGGL((sdpa_kernel<DP, true, false, false>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((sdpa_kernel<DP, false, false, false>), grid, block, 0, s, a);
   }
   return launch_status();
 }

@@ -29,6 +29,11 @@ DT_EXPORT size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int3
     bytes += align256((size_t)B * Skv * Hk * D * 2);
   }
   if (fused_out_proj) bytes += align256((size_t)B * Sq * Hq * D * 2);
+  // Optional part: room for the key-split form of the kernel (partial results of the pieces and the per-task
+  // counters), for launches whose workgroup count leaves a good part of the last round of compute units idle.  A
+  // call that is handed less than this, but at least the staging bytes above, runs unsplit.
+  SdpaSplit plan;
+  if (sdpa_split_plan(B, Hq, D, Sq, Skv, &plan)) bytes += align256(plan.bytes());
   return bytes;
 }
 
@@ -39,7 +44,7 @@ struct SdpaShape {
   int64_t Sq = 0, Skv = 0;
   bool prep = false;   // some segment is normalised or rotated on the way in
   bool empty = false;  // nothing to compute (no batch or no query row)
-  size_t need = 0;     // staging bytes, by the rule of dt_sdpa_workspace_bytes
+  size_t need = 0;     // staging bytes the request cannot run without (the first part of dt_sdpa_workspace_bytes)
 };
 
 // Argument checks shared by dt_sdpa_f16 and dt_sdpa_f16_static; touches no device state.
@@ -77,7 +82,8 @@ static dt_status sdpa_validate(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int
     if (k_seg[i].len > 0 && (!view_ok(k_seg[i].view, 8) || !view_ok(v_seg[i].view, 8))) return DT_INVALID;
   if (!o.ptr || (reinterpret_cast<uintptr_t>(o.ptr) & 7) || o.stride_b % 4 || o.stride_s % 4) return DT_INVALID;
   if (!Wo && o.stride_h % 4) return DT_INVALID;
-  sh.need = dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, prep ? 1 : 0, Wo ? 1 : 0);
+  if (prep) sh.need += align256((size_t)B * Sq * Hq * D * 2) + align256((size_t)B * Skv * Hk * D * 2);
+  if (Wo) sh.need += align256((size_t)B * Sq * Hq * D * 2);
   return DT_OK;
 }
 
@@ -200,8 +206,22 @@ static dt_status sdpa_enqueue(dt_stream stream, int32_t B, int32_t Hq, int32_t H
     }
   }
 
+  // What is left of the workspace behind the staging buffers takes the key-split form's partial results, if the
+  // launch is one that splitting helps and the room is there.
+  auto plan_split = [&](uint8_t* free_ws) {
+    SdpaSplit plan;
+    if (!workspace || !sdpa_split_plan(B, Hq, D, Sq, Skv, &plan)) return;
+    const size_t used = (size_t)(free_ws - static_cast<uint8_t*>(workspace));
+    if (workspace_bytes < used + plan.bytes() || (reinterpret_cast<uintptr_t>(workspace) & 255)) return;
+    a.counters = reinterpret_cast<int32_t*>(free_ws);
+    a.partials = reinterpret_cast<float*>(free_ws + plan.counter_bytes);
+    a.units = plan.units;
+    a.split_workgroups = plan.workgroups;
+  };
   if (Wo) {
     uint16_t* ow = reinterpret_cast<uint16_t*>(ws);
+    ws += align256((size_t)B * Sq * Hq * D * 2);
+    plan_split(ws);
     a.o = ow;
     a.o_sb = Sq * Hq * D;
     a.o_ss = (int64_t)Hq * D;
@@ -227,6 +247,7 @@ static dt_status sdpa_enqueue(dt_stream stream, int32_t B, int32_t Hq, int32_t H
     }
     return DT_OK;
   }
+  plan_split(ws);
   a.o = static_cast<uint16_t*>(o.ptr);
   a.o_sb = o.stride_b;
   a.o_ss = o.stride_s;
@@ -286,12 +307,15 @@ DT_EXPORT dt_status dt_sdpa_f16_static(dt_stream stream, int32_t B, int32_t Hq, 
     return st;
   if (sh.empty) return DT_OK;
   if (sh.need > (size_t)DT_SDPA_STATIC_SCRATCH_BYTES) return DT_OOM;  // beyond the fixed array: use dt_sdpa_f16
+  if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
+  // the staging bytes are a must; the key-split form's room is used if the array still has it
+  size_t give = dt_sdpa_workspace_bytes(B, Hq, Hk, D, sh.Sq, sh.Skv, sh.prep ? 1 : 0, Wo ? 1 : 0);
+  if (give > (size_t)DT_SDPA_STATIC_SCRATCH_BYTES) give = sh.need;
   void* ws = nullptr;
-  if (sh.need > 0) {
-    if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
+  if (give > 0) {
     ws = sdpa_static_scratch();
     if (!ws) return DT_DEVICE_ERROR;
   }
   return sdpa_enqueue(stream, B, Hq, Hk, D, n_qseg, q_seg, n_kvseg, k_seg, v_seg, rot_q, rot_k, eps, o, scale, Wo, bo,
-                      ws, sh.need, sh);
+                      ws, give, sh);
 }

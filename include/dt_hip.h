@@ -309,8 +309,18 @@ dt_status dt_qk_norm_rope_f16(dt_stream stream, dt_view4 x, int32_t B, int64_t S
  *             Models/UNet.swift:143-155): o is then [B, Sq, Hq*D] written with
  *             o.stride_s as row stride (stride_h unused), Wo fp16 [Hq*D, Hq*D]
  *             in [out, in] order, bo [Hq*D] or NULL
- *   workspace : device scratch of at least dt_sdpa_workspace_bytes(...) bytes,
- *             256-byte aligned; may be NULL when that function returns 0
+ *   workspace : device scratch, 256-byte aligned; may be NULL when nothing is
+ *             staged.  dt_sdpa_workspace_bytes(...) is the staging this call
+ *             cannot run without (fused_prep / fused_out_proj; less than that
+ *             is DT_OOM) plus, for launches that would occupy well under one
+ *             round of the card's compute units, room for the key-split form of
+ *             the kernel (each task's key tiles shared out over several
+ *             workgroups, fp32 partial results folded in a fixed order by the
+ *             piece that finishes last).  Given only the staging part, or
+ *             nothing, such a launch runs unsplit: same results to within one
+ *             rounding of the fp16 output, lower occupancy.
+ *             Environment: DT_SDPA_KEY_SPLIT=never|always overrides the
+ *             estimate (read at every call; for tests and measurements).
  * D in {40, 64, 128} (any D <= 128 that is a multiple of 8).
  * Inputs are expected to be finite.  A key whose V row holds Inf or NaN makes every output row of its (batch,
  * head) non-finite in the reference too, except where its probability underflows to zero; here such a V row can
@@ -324,9 +334,10 @@ dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32
                       float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
                       size_t workspace_bytes);
 
-/* Scratch dt_sdpa_f16 needs: room for normalised / rotated copies of Q and K
- * when `fused_prep` != 0 (any gamma or rot given) and for the attention output
- * when `fused_out_proj` != 0. */
+/* Scratch for dt_sdpa_f16: room for normalised / rotated copies of Q and K
+ * when `fused_prep` != 0 (any gamma or rot given), for the attention output
+ * when `fused_out_proj` != 0, and -- optional, see `workspace` above -- for the
+ * key-split form's partial results on the calling thread's current device. */
 size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int64_t Sq,
                                int64_t Skv, int32_t fused_prep, int32_t fused_out_proj);
 
@@ -337,8 +348,9 @@ size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int
  * it calls nothing that allocates or frees.
  *   The scratch is one fixed array of DT_SDPA_STATIC_SCRATCH_BYTES per GPU, resident on every GPU the library runs
  *   on until the process ends (its device address is looked up once per device, by dt_init or by the first call
- *   with that device current).  A request whose dt_sdpa_workspace_bytes() exceeds it returns DT_OOM and enqueues
- *   nothing: use dt_sdpa_f16 with a workspace of the caller's then.  The limit covers the fused QK-norm / RoPE
+ *   with that device current).  A request whose staging exceeds it returns DT_OOM and enqueues nothing: use
+ *   dt_sdpa_f16 with a workspace of the caller's then.  (The optional key-split room is used when the array still
+ *   has it, exactly as dt_sdpa_f16 uses a workspace of dt_sdpa_workspace_bytes().)  The limit covers the fused QK-norm / RoPE
  *   staging of a joint sequence of 4608 tokens x 24 heads x 128 (56.6 MB) and the fused unify-heads staging of
  *   SD 1.5 (5.2 MB).
  *   All calls on one GPU share that GPU's array, whose contents are whatever the last call left (every byte a

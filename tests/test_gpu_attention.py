@@ -620,3 +620,100 @@ def test_sdpa_wan_causal_chunked_windows(dthip, oracle, torch_cuda):
     # the windows matter: the first chunk's rows differ from full (non-causal) attention over all frames
     full = oracle.C.sdpa(np.ascontiguousarray(q[:, :frames]), k, v, scale)
     assert float(np.abs(full.astype(np.float32) - got[:, :frames].astype(np.float32)).max()) > 1e-2
+
+
+# ------------------------------------------------------------------ K3, key-split form
+
+SPLIT_CASES = [
+    # B, Sq, Skv, Hq, Hk, D, scale sign
+    (1, 300, 1000, 2, 2, 128, 1),     # ragged queries and keys, tasks cut into up to 8 pieces
+    (2, 256, 640, 3, 3, 128, 1),      # whole tiles; runs that span several tasks
+    (1, 70, 777, 8, 8, 40, 1),        # head size 40 (padded to 64)
+    (1, 130, 1900, 4, 2, 64, 1),      # grouped heads
+    (1, 520, 2100, 1, 1, 128, -1),    # a scale the kernel folds into the scores first (negative)
+    (1, 1, 300, 1, 1, 128, 1),        # one query row, five key tiles in two pieces
+]
+
+
+@pytest.mark.parametrize("B,Sq,Skv,Hq,Hk,D,sign", SPLIT_CASES)
+def test_sdpa_key_split_vs_oracle(dthip, oracle, torch_cuda, monkeypatch, B, Sq, Skv, Hq, Hk, D, sign):
+    """The key-split form of the kernel (a task's key tiles shared out over several workgroups, partial results
+    folded by the piece that finishes last), forced on small shapes: against the oracle, against the unsplit
+    kernel, and twice in a row (the fold order is fixed, so the result may not depend on the order of arrival)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(B * 1000 + Sq + Skv + D)
+    q, k, v = rand_qkv(rng, B, Sq, Skv, Hq, Hk, D)
+    scale = sign / np.sqrt(D)
+    want = oracle.C.sdpa(q, k, v, scale)
+    qd, kd, vd = (to_dev(torch, t) for t in (q, k, v))
+    monkeypatch.setenv("DT_SDPA_KEY_SPLIT", "always")
+    assert dthip.lib().dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, 0, 0) > 0  # the split is in force
+    print("sdpa key split", B, Sq, Skv, Hq, Hk, D, sign, flush=True)
+    got = dthip.sdpa_segments([qd], [kd], [vd], scale)
+    again = dthip.sdpa_segments([qd], [kd], [vd], scale)
+    monkeypatch.setenv("DT_SDPA_KEY_SPLIT", "never")
+    assert dthip.lib().dt_sdpa_workspace_bytes(B, Hq, Hk, D, Sq, Skv, 0, 0) == 0
+    plain = dthip.sdpa_segments([qd], [kd], [vd], scale)
+    torch.cuda.synchronize()
+    mx, rr = oracle.err_stats(got.cpu().numpy(), want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+    assert torch.equal(got, again)
+    # same arithmetic up to the fp32 fold of the pieces: a rounding step of the fp16 result at most
+    assert float((got.float() - plain.float()).abs().max()) <= 2e-3
+
+
+def test_sdpa_key_split_joint_segments_fused_prep(dthip, oracle, torch_cuda, monkeypatch):
+    """Key-split with text || image segments, fused per-head RMSNorm + RoPE staging and the static-scratch entry
+    point: all three forms agree bit for bit with each other and with the oracle within the attention bar."""
+    torch = torch_cuda
+    rng = np.random.default_rng(431)
+    T, h, w, H, D = 70, 24, 20, 3, 128
+    HW = h * w
+    segs = {n: (f16(rng.standard_normal((1, T, H, D))), f16(rng.standard_normal((1, HW, H, D)))) for n in "qkv"}
+    gam = {n: (f16(1 + 0.05 * rng.standard_normal(D)), f16(1 + 0.05 * rng.standard_normal(D))) for n in "qk"}
+    rot = f16(dthip.Flux1RotaryPositionEmbedding(h, w, T, channels=D))
+    scale = 1 / np.sqrt(D)
+    dev = lambda a: to_dev(torch, a)
+    args = dict(q_segs=[dev(t) for t in segs["q"]], k_segs=[dev(t) for t in segs["k"]],
+                v_segs=[dev(t) for t in segs["v"]], scale=scale, gamma_q=[dev(g) for g in gam["q"]],
+                gamma_k=[dev(g) for g in gam["k"]], rot_q=dev(rot), rot_k=dev(rot))
+
+    def prep(n):
+        parts = [oracle.C.rmsnorm(segs[n][i][0], gam[n][i], 1e-6) for i in range(2)]
+        return oracle.C.cmul(np.concatenate(parts, axis=0), rot)[None]
+
+    want = oracle.C.sdpa(prep("q"), prep("k"), np.concatenate(segs["v"], axis=1), scale)
+    monkeypatch.setenv("DT_SDPA_KEY_SPLIT", "always")
+    print("sdpa key split, joint segments with fused prep", flush=True)
+    got = dthip.sdpa_segments(**args)
+    got_static = dthip.sdpa_segments(**args, static_scratch=True)
+    # without the staging pass: two segments straight into the split kernel
+    plain_args = dict(q_segs=args["q_segs"], k_segs=args["k_segs"], v_segs=args["v_segs"], scale=scale)
+    seg_split = dthip.sdpa_segments(**plain_args)
+    monkeypatch.setenv("DT_SDPA_KEY_SPLIT", "never")
+    seg_plain = dthip.sdpa_segments(**plain_args)
+    torch.cuda.synchronize()
+    mx, rr = oracle.err_stats(got.cpu().numpy(), want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+    assert torch.equal(got, got_static)
+    assert float((seg_split.float() - seg_plain.float()).abs().max()) <= 2e-3
+
+
+def test_sdpa_key_split_by_its_own_estimate(dthip, oracle, torch_cuda, monkeypatch):
+    """A launch that fills a quarter of the card (4 heads x 4096 tokens: 64 workgroups of 64 key tiles) is split
+    without being told to; sampled rows against the oracle."""
+    torch = torch_cuda
+    monkeypatch.delenv("DT_SDPA_KEY_SPLIT", raising=False)
+    B, S, H, D = 1, 4096, 4, 128
+    assert dthip.lib().dt_sdpa_workspace_bytes(B, H, H, D, S, S, 0, 0) > 0
+    assert dthip.lib().dt_sdpa_workspace_bytes(1, 24, 24, D, 4608, 4608, 0, 0) == 0  # the Flux shape is not
+    rng = np.random.default_rng(4096)
+    q, k, v = rand_qkv(rng, B, S, S, H, H, D)
+    scale = 1 / np.sqrt(D)
+    print("sdpa key split by estimate", flush=True)
+    got = dthip.sdpa_segments([to_dev(torch, q)], [to_dev(torch, k)], [to_dev(torch, v)], scale).cpu().numpy()
+    rows = np.sort(rng.choice(S, size=40, replace=False))
+    rows[0], rows[-1] = 0, S - 1
+    want = oracle.C.sdpa(np.ascontiguousarray(q[:, rows]), k, v, scale)
+    mx, rr = oracle.err_stats(got[:, rows], want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
