@@ -283,7 +283,11 @@ static dt_status run_group(hipStream_t s, const HostGroup& h) {
     const bool big = (((M >= 1024) && (n_rows0 >= 256) && big_tiles >= kFillTiles) && pal_fits_big) || any_fused;
     // few token rows: halve the token tile so that more workgroups share the work
     const bool narrow = big && M < 1024;
-    const int BM = big ? (narrow ? 128 : 256) : 128, BN = big ? 256 : 128;
+    // palettes that only fit beside a 128-feature tile, and enough work for tall tiles: 256 tokens x 128 features
+    // (twice the MFMAs per unpacked weight of the 128 x 128 tile)
+    const bool tall = !big && !pal_fits_big && (w0.qbits == 7 || w0.qbits == 8) && M >= 1024 && n_rows0 >= 128 &&
+                      big_tiles * 2 >= kFillTiles;
+    const int BM = big ? (narrow ? 128 : 256) : (tall ? 256 : 128), BN = big ? 256 : 128;
     DenseArgs a;
     DenseGroup& g = a.g[0];
     g.x = h.X;
@@ -307,7 +311,8 @@ static dt_status run_group(hipStream_t s, const HostGroup& h) {
     a.total_tiles = g.tiles_m * tiles_n;
     finish_args(a, 1, cnt, K, w0);
     const int mode = choose_pal_mode(w0.qbits, a.nib, K, BM, BN);
-    dt_status st = launch_dense(s, a, !big ? kTile128x128 : narrow ? kTile128x256 : kTile256x256, w0.qbits, mode);
+    dt_status st = launch_dense(s, a, tall ? kTile256x128 : !big ? kTile128x128 : narrow ? kTile128x256 : kTile256x256,
+                                w0.qbits, mode);
     if (st != DT_OK) return st;
     for (int j = first; j < i; j++)
       if (h.wants_epi(j) && !(big && h.fusable(j))) {

@@ -14,9 +14,10 @@ constexpr int kMaxWeights = 8;
 constexpr int kMaxGroups = 4;
 constexpr int BK = 32;
 constexpr int kPalLdsBytes = 32768;
-// LDS a tile shape can spare for palettes: the 128 x 128 tile's X slots and weight ring are a quarter of the
-// 256 x 256 tile's, which leaves room for a per-row table of 256-entry palettes (128 rows x 512 B).
-constexpr int pal_lds_bytes(int BM, int BN) { return (BM == 128 && BN == 128) ? 65536 : kPalLdsBytes; }
+// LDS a tile shape can spare for palettes: the tiles of 128 features have a weight ring half the size of the
+// 256-feature tiles' (and the 128 x 128 tile X slots half the size too), which leaves room for a per-row table of
+// 256-entry palettes (128 rows x 512 B = 64 KB; with 256 tokens: 64 KB of X slots + 24 KB of ring + 64 KB = 152 KB).
+constexpr int pal_lds_bytes(int BM, int BN) { return BN == 128 ? 65536 : kPalLdsBytes; }
 
 enum PalMode : int {
   kPalShared = 0,  // palettes of every block the tile's rows touch, loaded once, slot = block - first block
@@ -496,8 +497,13 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const bool second = wave >= 4;     // unpacks weights 16..31 of its row's granule (waves 0-3: weights 0..15)
-  const int lt = tid & 255;
+  // Weight staging: two threads per weight row, each unpacking half of the row's 32-index granule.  With 256 rows
+  // that is every thread: waves 0-3 take weights 0..15 of rows 0..255, waves 4-7 weights 16..31.  With 128 rows it
+  // is half of them, and the four waves that stage are one per SIMD (waves 0-3: rows 64 * (wave % 2) + lane, half
+  // wave / 2); waves 4-7 only run MFMAs and the X transfers.
+  const bool second = BN == 256 ? wave >= 4 : ((wave >> 1) & 1) != 0;
+  const bool stager = BN == 256 || __builtin_amdgcn_readfirstlane(wave) < 4;  // wave-uniform
+  const int lt = BN == 256 ? (tid & 255) : (lane + 64 * (wave & 1));
   const int wn = wave & 1, wm = ((wave >> 1) & 1) | ((wave >> 2) << 1);  // waves w and w+4 share a SIMD and take different m slices
 
   // Tile order: bands of 4 token tiles; inside a band feature tiles outermost,
@@ -608,6 +614,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // they ask for.  Each of a row's two threads keeps half of the row's column current.
   const int pal_col = (b_row >> 7) * (256 << Q) + (b_row & 63) * 4 + ((b_row >> 6) & 1) * 2;  // byte offset of this row's column
   auto fill_pal_column = [&](int64_t blk) {
+    if (!stager) return;
     constexpr int ND = (1 << Q) / 4;  // dwords of palette per thread
     const uint32_t* src =
         reinterpret_cast<const uint32_t*>(w.data + palette_offset(lay, blk)) + (second ? ND : 0);
@@ -661,6 +668,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   int issued = 0;  // tiles loaded so far
   auto issue_idx = [&](IdxSet& R) {
     if constexpr (MODE != kPlainF16) {
+      if (!stager) return;
       const uint32_t* src = reinterpret_cast<const uint32_t*>(wbase + cur.off);
 #pragma unroll
       for (int i = 0; i < HW; i++) R.b[i] = src[i];
@@ -691,6 +699,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // piece 0 also turns the index dwords into a bit string; piece p yields offsets 4p .. 4p+3
   auto unpack_piece = [&](IdxSet& R, int p) {
     if constexpr (MODE != kPlainF16) {
+      if (!stager) return;
       if (p == 0) {
         own_bits<Q, HW>(R.b, second, be);
         if constexpr (MODE == kPalRow) pal_base = (uint32_t)pal_col;
@@ -703,6 +712,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     }
   };
   auto lookup = [&](int j) {
+    if (!stager) return;
     if constexpr (MODE == kPalGlobal)
       la[j] = *reinterpret_cast<const uint16_t*>(gpal + la[j]);
     else if constexpr (MODE != kPlainF16)
@@ -717,6 +727,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   const uint32_t w_dst = lds_address(Bs) + 2u * (uint32_t)w_chunk(b_row, second ? 2 : 0);
   auto write_weights = [&](int stage, int h) {
     if constexpr (MODE != kPlainF16) {
+      if (!stager) return;
       const uint4_t v = {la[8 * h] | (la[8 * h + 1] << 16), la[8 * h + 2] | (la[8 * h + 3] << 16),
                          la[8 * h + 4] | (la[8 * h + 5] << 16), la[8 * h + 6] | (la[8 * h + 7] << 16)};
       const uint32_t addr = w_dst + (uint32_t)(stage * B_STAGE * 2) + (uint32_t)(h * BN * 16);
@@ -734,6 +745,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   // Makes the wait for an index load happen here rather than at its first use.
   auto touch = [&](IdxSet& R) {
     if constexpr (MODE != kPlainF16) {
+      if (!stager) return;
 #pragma unroll
       for (int j = 0; j < HW; j++) asm volatile("" : "+v"(R.b[j]));
     }

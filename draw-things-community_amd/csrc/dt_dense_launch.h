@@ -5,7 +5,9 @@
 namespace dt {
 
 // Tile shapes the host side chooses between.
-enum DenseTile : int { kTile128x128 = 0, kTile128x256 = 1, kTile256x256 = 2 };
+// (tokens x features; 256 x 128 exists for the palettes that only fit beside a 128-feature tile -- per-row tables of
+// 128 and 256 entries -- and is instantiated for those index widths only)
+enum DenseTile : int { kTile128x128 = 0, kTile128x256 = 1, kTile256x256 = 2, kTile256x128 = 3 };
 
 template <int Q, int BM, int BN, bool POST>
 static dt_status launch_tiled(hipStream_t s, const DenseArgs& a, int mode) {
@@ -34,6 +36,14 @@ static dt_status launch_dense_qp(hipStream_t s, const DenseArgs& a, int tile, in
   switch (tile) {
     case kTile128x128: return launch_tiled<Q, 128, 128, POST>(s, a, mode);
     case kTile128x256: return launch_tiled<Q, 128, 256, POST>(s, a, mode);
+    case kTile256x128:
+      if constexpr (Q == 7 || Q == 8) {
+        if (mode != kPalRow) return DT_NO_KERNEL;
+        hipLaunchKernelGGL((dense_qx_kernel<Q, 256, 128, kPalRow, POST>), dim3((unsigned)a.total_tiles), dim3(512), 0, s, a);
+        return launch_status();
+      } else {
+        return DT_NO_KERNEL;  // the host side picks this tile for 7- and 8-bit indices only
+      }
     default: return launch_tiled<Q, 256, 256, POST>(s, a, mode);
   }
 }

@@ -61,6 +61,9 @@ CASES = [
     (1300, 1024, 1024, 8, 4096),  # 256-entry palettes with small blocks: fit beside no big tile -> small tile, per-row table
     (1100, 520, 768, 8, 512),     # the same with several blocks per row (K % nib != 0), ragged edges
     (1100, 768, 512, 7, 1024),    # 128-entry palettes, two rows per block
+    (2600, 2304, 512, 8, 512),    # the same palettes with enough work for the 256-token x 128-feature tile; ragged M
+    (2560, 2500, 768, 8, 4096),   # that tile with K % nib != 0 and a ragged last feature tile
+    (3000, 2200, 512, 7, 1024),   # that tile with 128-entry palettes, ragged both ways
 ]
 
 
@@ -87,7 +90,8 @@ def test_dense_qx_vs_oracle(dthip, oracle, torch_cuda, M, N, K, q, nib):
 
 
 @pytest.mark.parametrize("q,nib,K,N", [(8, 16384, 256, 320), (6, 4096, 512, 256), (5, 1024, 2048, 256),
-                                       (4, 512, 1024, 300), (4, 512, 768, 128), (7, 8192, 128, 256)])
+                                       (4, 512, 1024, 300), (4, 512, 768, 128), (7, 8192, 128, 256),
+                                       (8, 4096, 1024, 6144)])  # (the last: 256 x 128 tile, per-row 256-entry tables)
 def test_effective_weights_bit_exact(dthip, oracle, torch_cuda, q, nib, K, N):
     """X = I_K makes Y = W^T exactly (one nonzero product per output, fp16-representable):
     the weights the fused kernel multiplies by are bit-for-bit the dequantized tensor."""
