@@ -866,7 +866,8 @@ def sdpa_segments(q_segs, k_segs, v_segs, scale, gamma_q=None, gamma_k=None, rot
         return arr
 
     qa, ka, va = segs(q_segs, gq), segs(k_segs, gk), segs(v_segs, [None] * nk)
-    prep = any(g is not None for g in list(gq) + list(gk)) or rot_q is not None or rot_k is not None
+    # only K is staged for a fused norm / rotation (the queries are handled inside the attention kernel)
+    prep = any(g is not None for g in gk) or rot_k is not None
     fused = Wo is not None
     if out is None:
         shape = (B, Sq, Hq * D) if fused else (B, Sq, Hq, D)

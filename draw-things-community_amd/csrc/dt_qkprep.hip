@@ -12,8 +12,6 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-__device__ __forceinline__ float round_h(float v) { return round_f16(v); }
-
 // normalise-rotate-scale one (re, im) pair that is already in registers
 __device__ __forceinline__ uint32_t finish_pair(float a, float b, float inv, const uint16_t* gamma, int p,
                                                 const uint16_t* rot_row, float post_scale) {
@@ -106,41 +104,6 @@ __global__ void __launch_bounds__(256) qk_prep_row_kernel(const QkPrepArgs a) {
 // ---- 16-byte forms ------------------------------------------------------------
 // The same arithmetic with every access a whole 16-byte chunk (8 elements = 4 complex pairs): used when the
 // head dimension is a multiple of 8 and every row, the table and the norm weight are 16-byte aligned.
-
-// normalise-rotate-scale the 8 elements of one chunk; g and r are the chunk's norm weights and table entries
-__device__ __forceinline__ uint4_t finish_chunk(const float (&x)[8], float inv, bool has_gamma, const uint4_t& g,
-                                                bool has_rot, const uint4_t& r, float post_scale) {
-  uint4_t out;
-#pragma unroll
-  for (int q = 0; q < 4; q++) {
-    float a = x[2 * q], b = x[2 * q + 1];
-    if (has_gamma) {
-      a = round_h(a * inv * (float)bits_to_half((uint16_t)g[q]));
-      b = round_h(b * inv * (float)bits_to_half((uint16_t)(g[q] >> 16)));
-    }
-    if (has_rot) {
-      const float c = (float)bits_to_half((uint16_t)r[q]), sn = (float)bits_to_half((uint16_t)(r[q] >> 16));
-      const float na = round_h(a * c - b * sn);
-      const float nb = round_h(a * sn + b * c);
-      a = na;
-      b = nb;
-    }
-    if (post_scale != 1.0f) {
-      a = round_h(a * post_scale);
-      b = round_h(b * post_scale);
-    }
-    out[q] = (uint32_t)half_to_bits((half_t)a) | ((uint32_t)half_to_bits((half_t)b) << 16);
-  }
-  return out;
-}
-
-__device__ __forceinline__ void unpack_chunk(const uint4_t& v, float (&x)[8]) {
-#pragma unroll
-  for (int q = 0; q < 4; q++) {
-    x[2 * q] = (float)bits_to_half((uint16_t)v[q]);
-    x[2 * q + 1] = (float)bits_to_half((uint16_t)(v[q] >> 16));
-  }
-}
 
 // Per-head norm (or none): LPR = D / 8 lanes (a power of two) per (b, s, h) row, 256 / LPR rows per pass of a
 // workgroup, kHeadPasses passes per thread with all their loads issued before the first use.

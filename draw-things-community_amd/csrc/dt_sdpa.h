@@ -20,6 +20,13 @@ struct SdpaArgs {
   uint16_t* o;
   int64_t o_sb, o_ss, o_sh;
   float scale_log2e;
+  // Optional per-head RMSNorm and RoPE rotation of the queries, applied to the query fragments on their way into
+  // registers (same arithmetic and rounding as the norm / rotate pass): q_gamma[i] is segment i's norm weight [D]
+  // or null, q_rot the table [joint query rows, D] or null.
+  const uint16_t* q_gamma[kMaxSeg];
+  const uint16_t* q_rot;
+  float q_eps;
+  int32_t q_prep;  // any of the above is set
   // Key-split launch (optional; partials == nullptr runs one workgroup per task): workspace for the pieces' partial
   // results and the per-task tile counters, sized and laid out by sdpa_split_plan().
   float* partials;

@@ -21,6 +21,7 @@
 #include <cstdlib>
 
 #include "dt_common.h"
+#include "dt_qkprep.h"
 #include "dt_sdpa.h"
 
 namespace dt {
@@ -174,13 +175,51 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
     for (int i = 1; i < kMaxSeg; i++)
       if (i < a.n_qseg && qi >= a.q[i].start) sg = i;
     const uint16_t* qp = a.q[sg].ptr + b * a.q[sg].sb + (qi - a.q[sg].start) * a.q[sg].ss + h * a.q[sg].sh;
+    uint4_t qraw[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       const int d0 = ks * 16 + hi * 8;
-      uint4_t v = uint4_t{0, 0, 0, 0};
-      if (d0 < D) v = *reinterpret_cast<const uint4_t*>(qp + d0);
-      qf[ks] = __builtin_bit_cast(half8_t, v);
+      qraw[ks] = uint4_t{0, 0, 0, 0};
+      if (d0 < D) qraw[ks] = *reinterpret_cast<const uint4_t*>(qp + d0);
     }
+    if (a.q_prep) {  // uniform
+      // RMSNorm over the head, then the rotation: the row's D elements sit in this lane and in lane ^ 32
+      const uint16_t* gam = a.q_gamma[sg];
+      const uint16_t* rrow = a.q_rot ? a.q_rot + qi * D : nullptr;
+      float inv = 1.f;
+      if (gam) {
+        float ss = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          float x[8];
+          unpack_chunk(qraw[ks], x);
+#pragma unroll
+          for (int e = 0; e < 8; e++) ss += x[e] * x[e];
+        }
+        ss = sum32(ss);
+        inv = 1.0f / sqrtf(ss / (float)D + a.q_eps);
+      }
+      auto chunk16 = [](const uint16_t* p) __attribute__((always_inline)) {
+        if ((reinterpret_cast<uintptr_t>(p) & 15) == 0) return *reinterpret_cast<const uint4_t*>(p);
+        uint4_t v;
+#pragma unroll
+        for (int q = 0; q < 4; q++) v[q] = (uint32_t)p[2 * q] | ((uint32_t)p[2 * q + 1] << 16);
+        return v;
+      };
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        const int d0 = ks * 16 + hi * 8;
+        if (d0 < D) {
+          float x[8];
+          unpack_chunk(qraw[ks], x);
+          const uint4_t g = gam ? chunk16(gam + d0) : uint4_t{0, 0, 0, 0};
+          const uint4_t r = rrow ? chunk16(rrow + d0) : uint4_t{0, 0, 0, 0};
+          qraw[ks] = finish_chunk(x, inv, gam != nullptr, g, rrow != nullptr, r, 1.0f);
+        }
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = __builtin_bit_cast(half8_t, qraw[ks]);
   }
 
   // ---- K / V tile loaders ------------------------------------------------

@@ -24,10 +24,8 @@ DT_EXPORT size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int3
   using namespace dt;
   if (B <= 0 || Hq <= 0 || Hk <= 0 || D <= 0 || Sq <= 0 || Skv <= 0) return 0;
   size_t bytes = 0;
-  if (fused_prep) {
-    bytes += align256((size_t)B * Sq * Hq * D * 2);
-    bytes += align256((size_t)B * Skv * Hk * D * 2);
-  }
+  // (the queries are normalised and rotated inside the attention kernel; only K is staged)
+  if (fused_prep) bytes += align256((size_t)B * Skv * Hk * D * 2);
   if (fused_out_proj) bytes += align256((size_t)B * Sq * Hq * D * 2);
   // Optional part: room for the key-split form of the kernel (partial results of the pieces and the per-task
   // counters), for launches whose workgroup count leaves a good part of the last round of compute units idle.  A
@@ -43,6 +41,8 @@ namespace dt {
 struct SdpaShape {
   int64_t Sq = 0, Skv = 0;
   bool prep = false;   // some segment is normalised or rotated on the way in
+  bool qprep = false;  // ... a query segment (done inside the attention kernel)
+  bool kprep = false;  // ... a key segment (staged into the workspace)
   bool empty = false;  // nothing to compute (no batch or no query row)
   size_t need = 0;     // staging bytes the request cannot run without (the first part of dt_sdpa_workspace_bytes)
 };
@@ -57,20 +57,23 @@ static dt_status sdpa_validate(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int
   if (n_qseg > kMaxSeg || n_kvseg > kMaxSeg) return DT_NO_KERNEL;
   if (D % 8 != 0 || D > 128) return DT_NO_KERNEL;
   int64_t Sq = 0, Skv = 0;
-  bool prep = rot_q || rot_k;
+  bool qprep = rot_q != nullptr, kprep = rot_k != nullptr;
   for (int i = 0; i < n_qseg; i++) {
     if (q_seg[i].len < 0) return DT_INVALID;
     Sq += q_seg[i].len;
-    prep = prep || q_seg[i].gamma;
+    qprep = qprep || q_seg[i].gamma;
   }
   for (int i = 0; i < n_kvseg; i++) {
     if (k_seg[i].len < 0 || k_seg[i].len != v_seg[i].len) return DT_INVALID;
     Skv += k_seg[i].len;
-    prep = prep || k_seg[i].gamma;
+    kprep = kprep || k_seg[i].gamma;
   }
+  const bool prep = qprep || kprep;
   sh.Sq = Sq;
   sh.Skv = Skv;
   sh.prep = prep;
+  sh.qprep = qprep;
+  sh.kprep = kprep;
   if (B == 0 || Sq == 0) {
     sh.empty = true;
     return DT_OK;
@@ -82,7 +85,7 @@ static dt_status sdpa_validate(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int
     if (k_seg[i].len > 0 && (!view_ok(k_seg[i].view, 8) || !view_ok(v_seg[i].view, 8))) return DT_INVALID;
   if (!o.ptr || (reinterpret_cast<uintptr_t>(o.ptr) & 7) || o.stride_b % 4 || o.stride_s % 4) return DT_INVALID;
   if (!Wo && o.stride_h % 4) return DT_INVALID;
-  if (prep) sh.need += align256((size_t)B * Sq * Hq * D * 2) + align256((size_t)B * Skv * Hk * D * 2);
+  if (kprep) sh.need += align256((size_t)B * Skv * Hk * D * 2);
   if (Wo) sh.need += align256((size_t)B * Sq * Hq * D * 2);
   return DT_OK;
 }
@@ -94,7 +97,6 @@ static dt_status sdpa_enqueue(dt_stream stream, int32_t B, int32_t Hq, int32_t H
                               dt_view4 o, float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
                               size_t workspace_bytes, const SdpaShape& sh) {
   const int64_t Sq = sh.Sq, Skv = sh.Skv;
-  const bool prep = sh.prep;
   if (sh.empty) return DT_OK;
   if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
 
@@ -115,67 +117,64 @@ static dt_status sdpa_enqueue(dt_stream stream, int32_t B, int32_t Hq, int32_t H
   a.Skv = Skv;
   a.scale_log2e = scale * 1.44269504088896340736f;
 
-  if (prep) {
-    // RMSNorm -> cmul staged into contiguous copies; V is read in place.
-    uint16_t* qw = reinterpret_cast<uint16_t*>(ws);
-    ws += align256((size_t)B * Sq * Hq * D * 2);
-    uint16_t* kw = reinterpret_cast<uint16_t*>(ws);
-    ws += align256((size_t)B * Skv * Hk * D * 2);
-    for (int pass = 0; pass < 2; pass++) {
-      const dt_seq_segment* seg = pass == 0 ? q_seg : k_seg;
-      const int n = pass == 0 ? n_qseg : n_kvseg;
-      const int H = pass == 0 ? Hq : Hk;
-      const int64_t S = pass == 0 ? Sq : Skv;
-      uint16_t* dst = pass == 0 ? qw : kw;
-      const uint16_t* rot = pass == 0 ? rot_q : rot_k;
-      int64_t pos = 0;
-      for (int i = 0; i < n; i++) {
-        if (seg[i].len == 0) continue;
-        QkPrepArgs p;
-        p.src = static_cast<const uint16_t*>(seg[i].view.ptr);
-        p.src_sb = seg[i].view.stride_b;
-        p.src_ss = seg[i].view.stride_s;
-        p.src_sh = seg[i].view.stride_h;
-        p.dst = dst + pos * H * D;
-        p.dst_sb = S * H * D;
-        p.dst_ss = (int64_t)H * D;
-        p.dst_sh = D;
-        p.B = B;
-        p.S = seg[i].len;
-        p.H = H;
-        p.D = D;
-        p.gamma = seg[i].gamma;
-        p.eps = eps;
-        p.norm_per_head = 1;
-        p.rot = rot;
-        p.rot_pos0 = pos;
-        p.post_scale = 1.0f;
-        dt_status st = qk_prep_launch(s, p);
-        if (st != DT_OK) return st;
-        pos += seg[i].len;
-      }
-    }
-    a.n_qseg = 1;
-    a.q[0] = SdpaSeg{qw, Sq * Hq * D, (int64_t)Hq * D, D, 0};
-    a.n_kvseg = 1;
-    a.k[0] = SdpaSeg{kw, Skv * Hk * D, (int64_t)Hk * D, D, 0};
-    for (int i = 1; i < kMaxSeg; i++) {
-      a.q[i] = a.q[0];
-      a.k[i] = a.k[0];
-    }
-  } else {
+  // Queries: read in place, segment by segment; their RMSNorm and rotation happen inside the attention kernel.
+  {
     int64_t pos = 0;
     int n = 0;
     for (int i = 0; i < n_qseg; i++) {
       if (q_seg[i].len == 0) continue;
       const dt_view4& v = q_seg[i].view;
+      a.q_gamma[n] = q_seg[i].gamma;
       a.q[n++] = SdpaSeg{static_cast<const uint16_t*>(v.ptr), v.stride_b, v.stride_s, v.stride_h, pos};
       pos += q_seg[i].len;
     }
     a.n_qseg = n;
-    for (int i = n; i < kMaxSeg; i++) a.q[i] = a.q[0];
-    pos = 0;
-    n = 0;
+    for (int i = n; i < kMaxSeg; i++) {
+      a.q[i] = a.q[0];
+      a.q_gamma[i] = a.q_gamma[0];
+    }
+    a.q_rot = rot_q;
+    a.q_eps = eps;
+    a.q_prep = sh.qprep ? 1 : 0;
+  }
+  // Keys: RMSNorm -> cmul staged into one contiguous copy when asked for (the kernel moves K tiles from memory
+  // straight into LDS, so there is no register stage to do it in); otherwise read in place.  V is read in place.
+  const bool kprep = sh.kprep;
+  if (kprep) {
+    uint16_t* kw = reinterpret_cast<uint16_t*>(ws);
+    ws += align256((size_t)B * Skv * Hk * D * 2);
+    int64_t pos = 0;
+    for (int i = 0; i < n_kvseg; i++) {
+      if (k_seg[i].len == 0) continue;
+      QkPrepArgs p;
+      p.src = static_cast<const uint16_t*>(k_seg[i].view.ptr);
+      p.src_sb = k_seg[i].view.stride_b;
+      p.src_ss = k_seg[i].view.stride_s;
+      p.src_sh = k_seg[i].view.stride_h;
+      p.dst = kw + pos * Hk * D;
+      p.dst_sb = Skv * Hk * D;
+      p.dst_ss = (int64_t)Hk * D;
+      p.dst_sh = D;
+      p.B = B;
+      p.S = k_seg[i].len;
+      p.H = Hk;
+      p.D = D;
+      p.gamma = k_seg[i].gamma;
+      p.eps = eps;
+      p.norm_per_head = 1;
+      p.rot = rot_k;
+      p.rot_pos0 = pos;
+      p.post_scale = 1.0f;
+      dt_status st = qk_prep_launch(s, p);
+      if (st != DT_OK) return st;
+      pos += k_seg[i].len;
+    }
+    a.n_kvseg = 1;
+    a.k[0] = SdpaSeg{kw, Skv * Hk * D, (int64_t)Hk * D, D, 0};
+    for (int i = 1; i < kMaxSeg; i++) a.k[i] = a.k[0];
+  } else {
+    int64_t pos = 0;
+    int n = 0;
     for (int i = 0; i < n_kvseg; i++) {
       if (k_seg[i].len == 0) continue;
       const dt_view4& v = k_seg[i].view;
@@ -195,7 +194,7 @@ static dt_status sdpa_enqueue(dt_stream stream, int32_t B, int32_t Hq, int32_t H
       pos += v_seg[i].len;
     }
     for (int i = n; i < kMaxSeg; i++) a.v[i] = a.v[0];
-    if (prep && n > 1) {
+    if (kprep && n > 1) {
       // K was staged as one segment; the V segments keep their own table
       a.n_kvseg = n;
       for (int i = 1; i < n; i++) {

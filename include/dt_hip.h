@@ -334,8 +334,9 @@ dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32
                       float scale, const uint16_t* Wo, const uint16_t* bo, void* workspace,
                       size_t workspace_bytes);
 
-/* Scratch for dt_sdpa_f16: room for normalised / rotated copies of Q and K
- * when `fused_prep` != 0 (any gamma or rot given), for the attention output
+/* Scratch for dt_sdpa_f16: room for the normalised / rotated copy of K when
+ * `fused_prep` != 0 (any gamma or rot given; the queries are normalised and
+ * rotated inside the attention kernel and need none), for the attention output
  * when `fused_out_proj` != 0, and -- optional, see `workspace` above -- for the
  * key-split form's partial results on the calling thread's current device. */
 size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int64_t Sq,
@@ -350,9 +351,9 @@ size_t dt_sdpa_workspace_bytes(int32_t B, int32_t Hq, int32_t Hk, int32_t D, int
  *   on until the process ends (its device address is looked up once per device, by dt_init or by the first call
  *   with that device current).  A request whose staging exceeds it returns DT_OOM and enqueues nothing: use
  *   dt_sdpa_f16 with a workspace of the caller's then.  (The optional key-split room is used when the array still
- *   has it, exactly as dt_sdpa_f16 uses a workspace of dt_sdpa_workspace_bytes().)  The limit covers the fused QK-norm / RoPE
- *   staging of a joint sequence of 4608 tokens x 24 heads x 128 (56.6 MB) and the fused unify-heads staging of
- *   SD 1.5 (5.2 MB).
+ *   has it, exactly as dt_sdpa_f16 uses a workspace of dt_sdpa_workspace_bytes().)  The limit covers the staged K of a joint
+ *   sequence of 4608 tokens x 24 heads x 128 with fused QK-norm / RoPE (28.3 MB; up to ~10900 such tokens) and the
+ *   fused unify-heads staging of SD 1.5 (5.2 MB).
  *   All calls on one GPU share that GPU's array, whose contents are whatever the last call left (every byte a
  *   call reads it has written first): calls that may overlap in time on one GPU -- different streams, or different
  *   threads -- race on it and must be ordered by the caller.  Calls on one stream are ordered by the stream.

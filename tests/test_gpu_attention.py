@@ -250,6 +250,48 @@ def test_sdpa_fused_norm_rope_joint(dthip, oracle, torch_cuda):
     assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
 
 
+@pytest.mark.parametrize("B,Sq,Skv,Hq,Hk,D,q_only,misalign", [
+    (2, 300, 77, 8, 8, 40, True, False),     # SD-style head size 40 (padded to 64 inside): norm on Q only, nothing staged
+    (1, 270, 530, 4, 2, 64, False, False),   # grouped heads, D = 64, norm + rotation on both sides, B = 1
+    (1, 513, 200, 2, 2, 128, True, True),    # norm weight and table not 16-byte aligned; rotation on Q only
+])
+def test_sdpa_fused_norm_rope_on_queries_in_kernel(dthip, oracle, torch_cuda, B, Sq, Skv, Hq, Hk, D, q_only, misalign):
+    """Per-head RMSNorm and rotation of the queries happen inside the attention kernel (on the query fragments in
+    registers), K goes through the staging pass only when it asks for it: against the oracle's RMSNorm -> cmul ->
+    attention chain, and -- with prep on the query side only -- with no workspace at all."""
+    torch = torch_cuda
+    rng = np.random.default_rng(Sq + D)
+    q, k, v = rand_qkv(rng, B, Sq, Skv, Hq, Hk, D)
+    gq, gk = f16(1 + 0.05 * rng.standard_normal(D)), f16(1 + 0.05 * rng.standard_normal(D))
+    use_rot = D % 16 == 0
+    n_pos = max(Sq, Skv)
+    rot = f16(dthip.WanRotaryPositionEmbedding(1, n_pos, 1, channels=D)) if use_rot else None
+    scale = 1 / np.sqrt(D)
+
+    def dev_off(a):
+        """On the device, at an address that is 4-byte but not 16-byte aligned when `misalign` asks for it."""
+        if not misalign:
+            return to_dev(torch, a)
+        flat = torch.zeros(a.size + 2, dtype=torch.float16, device="cuda")
+        flat[2:] = to_dev(torch, a).reshape(-1)
+        return flat[2:].view(*a.shape)
+
+    def prep(x, g, S):
+        y = np.stack([oracle.C.rmsnorm(x[b], g, 1e-6) for b in range(B)])
+        if use_rot:
+            y = np.stack([oracle.C.cmul(y[b], rot[:S]) for b in range(B)])
+        return y
+
+    want = oracle.C.sdpa(prep(q, gq, Sq), k if q_only else prep(k, gk, Skv), v, scale)
+    kw = dict(gamma_q=[dev_off(gq)], rot_q=None if rot is None else dev_off(rot))
+    if not q_only:
+        kw.update(gamma_k=[to_dev(torch, gk)], rot_k=None if rot is None else to_dev(torch, rot))
+    print("sdpa fused prep on queries", B, Sq, Skv, Hq, Hk, D, q_only, misalign, flush=True)
+    got = dthip.sdpa_segments([to_dev(torch, q)], [to_dev(torch, k)], [to_dev(torch, v)], scale, **kw).cpu().numpy()
+    mx, rr = oracle.err_stats(got, want)
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
 def test_sdpa_fused_output_projection(dthip, oracle, torch_cuda):
     """SD1.5: multiHeadOutputProjectionFused -- the op owns W_o [HD, HD] and b_o and returns [B, S, HD]."""
     torch = torch_cuda

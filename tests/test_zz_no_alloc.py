@@ -10,7 +10,7 @@ MAX_ABS, REL_RMS = 2e-2, 1e-3
 
 
 def _case(dthip, oracle, torch, rng, T, h, w, H, D, fused_out):
-    """Joint text || image attention with fused per-head RMSNorm + RoPE (workspace: staged Q and K), or SD 1.5 style
+    """Joint text || image attention with fused per-head RMSNorm + RoPE (workspace: staged K), or SD 1.5 style
     attention with the fused unify-heads projection (workspace: staged attention output)."""
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
     f16 = lambda a: np.asarray(a, dtype=np.float16)
@@ -75,7 +75,7 @@ def test_static_scratch_entry_point_matches_workspace_entry_point(dthip, oracle,
 def test_static_scratch_rejects_requests_beyond_the_array(dthip):
     import torch
 
-    B, S, H, D = 1, 9000, 24, 128   # staged Q + K: 2 * 9000 * 24 * 128 * 2 B = 110 MB > 64 MiB
+    B, S, H, D = 1, 12000, 24, 128   # staged K: 12000 * 24 * 128 * 2 B = 73.7 MB > 64 MiB
     q = torch.zeros((B, S, H, D), dtype=torch.float16, device="cuda")
     g = torch.ones(D, dtype=torch.float16, device="cuda")
     assert dthip.lib().dt_sdpa_workspace_bytes(B, H, H, D, S, S, 1, 0) > dthip.STATIC_SCRATCH_BYTES
@@ -90,7 +90,7 @@ def test_static_scratch_rejects_requests_beyond_the_array(dthip):
 
 def test_static_scratch_at_the_documented_flux_shape(dthip):
     """The shape the array is sized for: 512 text + 64 x 64 image tokens, 24 heads x 128, fused per-head RMSNorm and
-    RoPE (staged Q and K: 56.6 MB, reaching the far end of the 64 MiB array) -- bit for bit against dt_sdpa_f16."""
+    RoPE (staged K: 28.3 MB of the 64 MiB array) -- bit for bit against dt_sdpa_f16."""
     import torch
 
     T, h, w, H, D = 512, 64, 64, 24, 128
@@ -122,7 +122,7 @@ def test_static_scratch_validates_like_the_workspace_entry_point(dthip):
 
     z = lambda *s: torch.zeros(s, dtype=torch.float16, device="cuda")
     g = torch.ones(128, dtype=torch.float16, device="cuda")
-    big = 9000  # staged Q + K beyond 64 MiB at 24 heads x 128
+    big = 12000  # staged K beyond 64 MiB at 24 heads x 128
     cases = [
         (dict(q_segs=[z(1, big, 24, 128)], k_segs=[z(1, big, 5, 128)], v_segs=[z(1, big, 5, 128)]), dthip.DT_INVALID),  # 5 does not divide 24
         (dict(q_segs=[z(1, big, 24, 136)], k_segs=[z(1, big, 24, 136)], v_segs=[z(1, big, 24, 136)]), dthip.DT_NO_KERNEL),  # D > 128
