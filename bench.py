@@ -2,10 +2,16 @@
 """Benchmark of the transformer-block hot path on one MI355X.
 
 A "step" is one pass of the Flux.1-dev-shape double-stream joint attention block's hot path
-(512 text + 4096 image tokens, 24 heads x 128, q6p weights): two fused-QKV palettized Dense launches
-(text M=512, image M=4096; three 3072->3072 weights each) whose epilogue applies the per-head QK RMSNorm and RoPE, joint
-ScaledDotProductAttention over 4608 tokens, and the two palettized output projections.
-All inputs are resident in HBM before the timed region.  Prints ONE JSON line.
+(512 text + 4096 image tokens, 24 heads x 128, q6p weights): the six fused-QKV palettized Dense projections
+(text M=512, image M=4096; three 3072->3072 weights each) as one grouped launch whose epilogue applies the per-head
+QK RMSNorm and RoPE, joint ScaledDotProductAttention over 4608 tokens, and the two palettized output projections as
+one grouped launch.  All inputs are resident in HBM before the timed region.  Prints ONE JSON line.
+
+The timed region launches the three kernels one by one with an event before and after each, so the line's
+per-kernel times ('kernels_in_step', and 'roofline') are means over the very steps that 'value' is computed from;
+'breakdown_consistent' says whether they add up to the step.  The single-kernel legs that follow
+('kernels_standalone_loops') repeat one launch back to back and are checked to run on the step's own data.  The CPU
+baseline leg runs the oracle on the step's own inputs and compares every output element ('step_checked').
 """
 import argparse
 import importlib
@@ -22,7 +28,7 @@ PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
 # counters read for a 256 MiB device copy (x2.00 and x1.00); the summary is profiles/bench_flux_block_counters.txt
-MEASURED_TRAFFIC_BYTES = {"dense_qkv": 3.742e8, "sdpa": 1.326e8}
+MEASURED_TRAFFIC_BYTES = {"dense_qkv": 3.742e8, "sdpa": 1.328e8}
 TRAFFIC_SOURCE = "profiles/bench_flux_block_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script; not measured by this run)"
 SDPA_NAME = "sdpa_kernel<128> S=4608 H=24"
 QKV_NAME = "dense_qx_kernel<6,256,256> M=4096+512 N=3x3072 K=3072 (fused norm/RoPE epilogue)"
@@ -104,6 +110,77 @@ def other_configs(pkg, torch, np):
     sdpa("cfg5 Wan self-attention H40 D128 S32760", 1, 32760, 32760, 40, 128, 2)
     sdpa("cfg5 Wan cross-attention H40 D128 Sq32760 Skv512", 1, 32760, 512, 40, 128, 3)
     dense("cfg5 Dense q5p M32760 5120->5120", 32760, 5120, [5120], "q5p", 2)
+    return out
+
+
+def occupancy_sweep(pkg, torch, np, sampler_cls):
+    """What the card delivers as a function of how many of its compute units a launch keeps busy: attention launches
+    of ONE round of workgroups (18 x heads workgroups of 72 key tiles each, 4608 tokens, head size 128) for a growing
+    number of heads, the two-round Flux launch, Dense launches of one, one and a half, two and three rounds of
+    256 x 256 tiles, and the key-split form of the attention kernel against the unsplit one -- each in a sustained
+    loop with the shader clock sampled from sysfs.  Answers whether the idle compute units of a launch's last round
+    are throughput lost (they are not, for attention: per-workgroup time grows by a third from half to full
+    occupancy while the clock falls by a fifth)."""
+    dev = "cuda"
+    out = {}
+
+    def timed(fn, flop, name, extra=None):
+        fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        while time.perf_counter() - t < 0.15:
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+        sampler = sampler_cls(torch)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n = 300
+        sampler.start()
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        clk = sampler.stop()
+        ms = e0.elapsed_time(e1) / n
+        out[name] = {"us": round(ms * 1e3, 1), "tflops": round(flop / ms / 1e9, 1),
+                     "sclk_mhz_median": None if clk is None else clk["median"]}
+        if extra:
+            out[name].update(extra)
+
+    S, D = 4608, 128
+    saved = os.environ.get("DT_SDPA_KEY_SPLIT")
+    for H in (2, 4, 7, 10, 12, 14, 24):
+        q, k, v = (torch.randn((1, S, H, D), device=dev).half() for _ in range(3))
+        o = torch.empty_like(q)
+        os.environ["DT_SDPA_KEY_SPLIT"] = "never"
+        timed(lambda: pkg.sdpa_segments([q], [k], [v], 1 / np.sqrt(D), out=o), 4.0 * H * S * S * D,
+              f"sdpa {H} heads x 4608 tokens, unsplit", {"workgroups": 18 * H, "key_tiles_each": 72})
+        if H in (4, 24):
+            os.environ["DT_SDPA_KEY_SPLIT"] = "always"
+            timed(lambda: pkg.sdpa_segments([q], [k], [v], 1 / np.sqrt(D), out=o), 4.0 * H * S * S * D,
+                  f"sdpa {H} heads x 4608 tokens, key-split into one equal run per compute unit",
+                  {"workgroups": 256, "key_tiles_each": round(18 * H * 72 / 256, 1)})
+    if saved is None:
+        os.environ.pop("DT_SDPA_KEY_SPLIT", None)
+    else:
+        os.environ["DT_SDPA_KEY_SPLIT"] = saved
+    rng = np.random.default_rng(0)
+
+    def synth(N, K, q, nib):
+        count = N * K
+        pal = (rng.standard_normal(((count + nib - 1) // nib, 1 << q)) * 0.02).astype(np.float16)
+        idx = rng.integers(0, 1 << q, size=count, dtype=np.uint8)
+        return pkg.QxTensor.from_packed(pkg.pack_qx(q, nib, pal, idx), q, nib, (N, K))
+
+    x = torch.randn(4096, 3072, device=dev).half()
+    for kind in ("q6p", "f16"):
+        for nt in (12, 16, 24, 32, 48):
+            N = 256 * nt
+            w = synth(N, 3072, 6, 4096) if kind == "q6p" else pkg.QxTensor.from_f16((torch.randn(N, 3072, device=dev) * 0.02).half())
+            y = torch.empty(4096, N, device=dev, dtype=torch.float16)
+            timed(lambda: pkg.dense_multi(x, [w], [None], outs=[y]), 2.0 * 4096 * 3072 * N,
+                  f"dense {kind} M4096 K3072 N{N}", {"tiles_256x256": 16 * nt, "rounds_of_256": round(16 * nt / 256, 2)})
     return out
 
 
@@ -234,6 +311,9 @@ def main():
     ap.add_argument("--clock-probe", action="store_true",
                     help="also run the two kernels of the step, the plain fp16 Dense and the vendor library's fp16 GEMM of the QKV shape for a few seconds each on random and on all-zero "
                          "activations while sampling the card's clock with rocm-smi (adds 'clock_probe' to the line)")
+    ap.add_argument("--occupancy-sweep", action="store_true",
+                    help="also time attention and Dense launches that keep a quarter ... all of the compute units busy, "
+                         "and the key-split attention kernel against the unsplit one (adds 'occupancy_sweep' to the line)")
     ap.add_argument("--other-configs", action="store_true",
                     help="also time the operators of the other benchmark configurations (SD 1.5, q8p Dense alone, "
                          "Flux at 2048 x 2048 with q4p, Wan 14B with q5p) and add them to the JSON line as 'other_configs'")
@@ -627,6 +707,7 @@ def main():
         }
 
     other = other_configs(pkg, torch, np) if args.other_configs else None
+    sweep = occupancy_sweep(pkg, torch, np, SclkSampler) if args.occupancy_sweep else None
     probe = None
     if args.clock_probe:
         saved = {}
@@ -676,6 +757,8 @@ def main():
     }
     if other is not None:
         line["other_configs"] = other
+    if sweep is not None:
+        line["occupancy_sweep"] = sweep
     if probe is not None:
         line["clock_probe"] = probe
     print(json.dumps(line))
