@@ -28,11 +28,36 @@ def test_host_only_entry_points(dthip, oracle):
         for count in (0, 1, nib - 1, nib, 5 * nib + 3, 3072 * 3072):
             assert dthip.qx_bytes(q, nib, count) == oracle.C.qx_bytes(q, nib, count)
     assert dthip.qx_bytes(3, 32, 10) == -1 and dthip.qx_bytes(9, 32, 10) == -1 and dthip.qx_bytes(6, 0, 10) == -1
-    # workspace sizing: nothing needed for the plain call, Q'+K' for the fused prep, O for the fused projection
+    # workspace sizing: nothing needed for the plain call, K' for the fused prep (the queries are normalised and
+    # rotated inside the kernel), O for the fused projection
     assert L.dt_sdpa_workspace_bytes(1, 24, 24, 128, 4608, 4608, 0, 0) == 0
     one = 4608 * 24 * 128 * 2
-    assert L.dt_sdpa_workspace_bytes(1, 24, 24, 128, 4608, 4608, 1, 0) == 2 * one
-    assert L.dt_sdpa_workspace_bytes(1, 24, 24, 128, 4608, 4608, 1, 1) == 3 * one
+    assert L.dt_sdpa_workspace_bytes(1, 24, 24, 128, 4608, 4608, 1, 0) == one
+    assert L.dt_sdpa_workspace_bytes(1, 24, 24, 128, 4608, 4608, 1, 1) == 2 * one
+
+
+def test_key_split_planning(dthip, monkeypatch):
+    """Which attention launches get room for the key-split form (host arithmetic; without a device the plan assumes
+    256 compute units): launches of whole or several rounds of workgroups never, launches well under one round with
+    enough key tiles do, and the environment knob overrides the estimate either way."""
+    L = dthip.lib()
+    ws = lambda B, H, D, Sq, Skv: L.dt_sdpa_workspace_bytes(B, H, H, D, Sq, Skv, 0, 0)
+    monkeypatch.delenv("DT_SDPA_KEY_SPLIT", raising=False)
+    assert ws(1, 24, 128, 4608, 4608) == 0         # 432 workgroups = 1.69 rounds: measured slower when split
+    assert ws(1, 24, 128, 16896, 16896) == 0       # 6.19 rounds
+    assert ws(2, 8, 40, 4096, 4096) == 0           # exactly one round
+    assert ws(2, 8, 40, 4096, 77) == 0             # two key tiles: nothing to cut
+    # 64 workgroups of 64 key tiles: one run per compute unit, two partial-result slots each, plus the counters
+    slot = (128 // 32 * 16 * 512 + 2 * 512) * 4
+    assert ws(1, 4, 128, 4096, 4096) == 256 + 2 * 256 * slot
+    # 8 workgroups: at most 8 pieces per task
+    assert ws(1, 1, 128, 2048, 16384) == 256 + 2 * 64 * slot
+    assert ws(1, 1, 64, 2048, 16384) == 256 + 2 * 64 * (64 // 32 * 16 * 512 + 2 * 512) * 4
+    monkeypatch.setenv("DT_SDPA_KEY_SPLIT", "never")
+    assert ws(1, 4, 128, 4096, 4096) == 0
+    monkeypatch.setenv("DT_SDPA_KEY_SPLIT", "always")
+    assert ws(1, 24, 128, 4608, 4608) == 1792 + 2 * 256 * slot   # 432 counters (1728 bytes), 256-byte aligned
+    assert ws(1, 1, 128, 1, 64) == 0                # a single key tile cannot be cut
 
 
 def test_missing_library_fails_loudly(dthip, monkeypatch):
