@@ -99,10 +99,10 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
   // Tiles go from memory straight into LDS.  A wave's transfer instruction
   // fills 1 KB of a tile, lane l landing on its 16-byte slot l; each thread
   // issues LOADS of them per K tile and per V tile and fetches the chunk that
-  // the swizzle assigns to its slot.  Lanes whose row lies past the last key,
-  // or whose chunk lies past D, stay idle: those slots keep what they held
-  // (zeros from the start, or an earlier tile's finite values), which the
-  // masked scores and the zero padding of Q make harmless.
+  // the swizzle assigns to its slot.  Lanes whose chunk lies past D stay idle
+  // (those slots keep the zeros they were given at the start), and so do, for
+  // K, lanes whose row lies past the last key (their scores are masked whatever
+  // the slot holds); V rows past the last key are zeroed (see zero_slot).
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   int ld_row[LOADS], k_ch[LOADS], v_ch[LOADS];
 #pragma unroll
@@ -272,11 +272,21 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) off[i] = (uint32_t)((ld_row[i] * c.ss + chs[i] * 8) * 2);
   };
+  // (zero_tail: rows of the tile past the last key get zeros instead of keeping an earlier tile's bytes -- for V,
+  // whose stale rows would otherwise meet a probability of exactly zero in the second MFMA: 0 x Inf = NaN)
+  auto zero_slot = [&](unsigned char* dst, int i) __attribute__((always_inline)) {
+    *reinterpret_cast<uint4_t*>(dst + (wave * LOADS + i) * 1024 + lane * 16) = uint4_t{0, 0, 0, 0};
+  };
   auto issue_general = [&](const SdpaSeg* segs, SegCursor& c, uint32_t (&off)[LOADS], const int (&chs)[LOADS],
-                           unsigned char* dst) __attribute__((always_inline)) {
+                           unsigned char* dst, bool zero_tail) __attribute__((always_inline)) {
     if (c.row0 < Skv) {
       if (c.row0 >= c.end) seek(segs, c, off, chs);  // uniform
       const int64_t last = c.row0 + BKV < Skv ? c.row0 + BKV : Skv;
+      if (zero_tail && last - c.row0 < BKV) {  // uniform: the ragged last tile
+#pragma unroll
+        for (int i = 0; i < LOADS; i++)
+          if (c.row0 + ld_row[i] >= Skv) zero_slot(dst, i);
+      }
       if (last <= c.end && c.ss > 0 && c.ss < (1 << 24)) {
         const int n_rows = (int)(last - c.row0);
         const void* base = c.base;
@@ -314,11 +324,16 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       }
       rows_left -= BKV;
     } else {
-      issue_general(a.k, kcur, k_off, k_ch, dst);
+      issue_general(a.k, kcur, k_off, k_ch, dst, false);
     }
   };
   auto issue_v = [&](unsigned char* dst) __attribute__((always_inline)) {
     if constexpr (ONESEG) {
+      if (rows_left_v < BKV) {  // uniform: the ragged last tile
+#pragma unroll
+        for (int i = 0; i < LOADS; i++)
+          if (ld_row[i] >= rows_left_v) zero_slot(dst, i);
+      }
 #pragma unroll
       for (int i = 0; i < LOADS; i++) {
         if (ld_row[i] < rows_left_v && v_ch[i] * 8 < D)
@@ -327,7 +342,7 @@ __global__ void __launch_bounds__(512) sdpa_kernel(const SdpaArgs a) {
       }
       rows_left_v -= BKV;
     } else {
-      issue_general(a.v, vcur, v_off, v_ch, dst);
+      issue_general(a.v, vcur, v_off, v_ch, dst, true);
     }
   };
   // ---- running state -----------------------------------------------------

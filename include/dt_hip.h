@@ -322,10 +322,10 @@ dt_status dt_qk_norm_rope_f16(dt_stream stream, dt_view4 x, int32_t B, int64_t S
  *             Environment: DT_SDPA_KEY_SPLIT=never|always overrides the
  *             estimate (read at every call; for tests and measurements).
  * D in {40, 64, 128} (any D <= 128 that is a multiple of 8).
- * Inputs are expected to be finite.  A key whose V row holds Inf or NaN makes every output row of its (batch,
- * head) non-finite in the reference too, except where its probability underflows to zero; here such a V row can
- * in addition reach rows through the unused slots of the ragged last key tile (probability exactly 0 there, and
- * 0 x Inf = NaN).  Non-finite Q / K scores behave as in the reference (the row's output is NaN).
+ * Inputs are expected to be finite.  A key whose V row holds Inf or NaN makes the output rows of its (batch, head)
+ * non-finite, as in the reference (probability x Inf, and 0 x Inf = NaN where the probability underflows); it
+ * reaches no other (batch, head), and the unused rows of the ragged last key tile are zeroed rather than left holding
+ * an earlier tile's values.  Non-finite Q / K scores behave as in the reference (the row's output is NaN).
  */
 dt_status dt_sdpa_f16(dt_stream stream, int32_t B, int32_t Hq, int32_t Hk, int32_t D,
                       int32_t n_qseg, const dt_seq_segment* q_seg, int32_t n_kvseg,
