@@ -331,8 +331,13 @@ class QxTensor:
 # --------------------------------------------------------------------------
 
 class GEMMFlag:
+    """Functional.GEMMFlag: permissions to compute at a given precision, not requests (Models/Flux1.swift:134, 162,
+    229-231).  `Int8` is what FlashAttentionLevel.quantized adds to an attention's flags (`[.Int8, .Float16]`,
+    Models/UNetProtocol.swift:14-19): this library computes such calls with its fp16 kernel (fp16 operands, fp32
+    accumulation and statistics), which every combination of these flags permits."""
     Float16 = 1
     Float32 = 2
+    Int8 = 4
 
 
 @dataclass

@@ -759,3 +759,19 @@ def test_sdpa_key_split_by_its_own_estimate(dthip, oracle, torch_cuda, monkeypat
     want = oracle.C.sdpa(np.ascontiguousarray(q[:, rows]), k, v, scale)
     mx, rr = oracle.err_stats(got[:, rows], want)
     assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+def test_sdpa_quantized_level_flags_are_permissions(dthip, oracle, torch_cuda):
+    """FlashAttentionLevel.quantized builds ScaledDotProductAttention(scale:, flags: [.Int8, .Float16])
+    (Models/Flux1.swift:228-232): the flags permit lower precision, they do not ask for it, so the call is served by
+    the fp16 kernel -- the same bits as with [.Float16], inside the attention bar of the oracle."""
+    torch = torch_cuda
+    rng = np.random.default_rng(229)
+    q, k, v = rand_qkv(rng, 1, 300, 520, 3, 3, 128)
+    scale = 1 / np.sqrt(128)
+    qd, kd, vd = (to_dev(torch, t) for t in (q, k, v))
+    f16_only = dthip.ScaledDotProductAttention(scale=scale, flags=dthip.GEMMFlag.Float16)(qd, kd, vd)
+    quantized = dthip.ScaledDotProductAttention(scale=scale, flags=dthip.GEMMFlag.Int8 | dthip.GEMMFlag.Float16)(qd, kd, vd)
+    assert torch.equal(f16_only, quantized)
+    mx, rr = oracle.err_stats(quantized.cpu().numpy(), oracle.C.sdpa(q, k, v, scale))
+    assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
