@@ -226,3 +226,76 @@ def test_dense_fused_heads_random_shapes(dthip, oracle, torch_cuda):
             tol = np.repeat(np.maximum(mag * 2.0 ** -9, 2.0 ** -14), 2, axis=-1)
             diff = np.abs(outs[j].cpu().numpy().reshape(M, H, hd).astype(np.float32) - wf)
             assert (diff <= tol).all(), (i, j, float((diff / tol).max()))
+
+
+def test_sdpa_segments_prep_and_key_split_random(dthip, oracle, torch_cuda, monkeypatch):
+    """Attention over random segment lists with every optional stage drawn at random -- per-segment norm weights on
+    the query side (applied inside the kernel) and on the key side (staged), rotation tables on either side, grouped
+    heads, head sizes from 8 to 128, positive and negative scales, the key-split form forced on, forced off or left
+    to the library's estimate, the caller's workspace or the static scratch -- against the oracle's
+    RMSNorm -> cmul -> attention chain."""
+    torch = torch_cuda
+    rng = np.random.default_rng(106)
+    for i in range(60):
+        D = int(rng.choice([40, 64, 128, 128, 128, 32, 16, 8, 24]))
+        Hk = int(rng.integers(1, 4))
+        Hq = Hk * int(rng.choice([1, 1, 2, 3]))
+        B = int(rng.choice([1, 1, 2]))
+        qlens = [int(rng.integers(1, 400)) for _ in range(int(rng.integers(1, 4)))]
+        klens = [int(rng.integers(1, 900)) for _ in range(int(rng.integers(1, 4)))]
+        Sq, Skv = sum(qlens), sum(klens)
+        q = [f16(rng.standard_normal((B, n, Hq, D))) for n in qlens]
+        k = [f16(rng.standard_normal((B, n, Hk, D))) for n in klens]
+        v = [f16(rng.standard_normal((B, n, Hk, D))) for n in klens]
+        use_gq, use_gk = rng.random() < 0.6, rng.random() < 0.4
+        gq = [f16(1 + 0.05 * rng.standard_normal(D)) if use_gq and rng.random() < 0.8 else None for _ in qlens]
+        gk = [f16(1 + 0.05 * rng.standard_normal(D)) if use_gk and rng.random() < 0.8 else None for _ in klens]
+        rot = f16(dthip.WanRotaryPositionEmbedding(1, max(Sq, Skv), 1, channels=D)) if D % 16 == 0 and rng.random() < 0.6 else None
+        rot_q = rot if rot is not None and rng.random() < 0.8 else None
+        rot_k = rot if rot is not None and rng.random() < 0.6 else None
+        scale = float(rng.choice([1 / np.sqrt(D), 0.07, -0.05]))
+        mode = str(rng.choice(["always", "never", "auto"]))
+        static = bool(rng.random() < 0.3)
+        if mode == "auto":
+            monkeypatch.delenv("DT_SDPA_KEY_SPLIT", raising=False)
+        else:
+            monkeypatch.setenv("DT_SDPA_KEY_SPLIT", mode)
+        print("sdpa segments", i, B, qlens, klens, Hq, Hk, D, use_gq, use_gk, rot_q is not None, rot_k is not None,
+              round(scale, 3), mode, static, flush=True)
+
+        def prep(parts, gs, r, S):
+            out = []
+            for b in range(B):
+                rows = np.concatenate([p[b] if g is None else oracle.C.rmsnorm(p[b], g, 1e-6) for p, g in zip(parts, gs)])
+                out.append(rows if r is None else oracle.C.cmul(rows, r[:S]))
+            return np.stack(out)
+
+        want = oracle.C.sdpa(prep(q, gq, rot_q, Sq), prep(k, gk, rot_k, Skv), np.concatenate(v, axis=1), scale)
+        dev = lambda a: None if a is None else to_dev(torch, a)
+        got = dthip.sdpa_segments([dev(t) for t in q], [dev(t) for t in k], [dev(t) for t in v], scale,
+                                  gamma_q=[dev(g) for g in gq] if any(g is not None for g in gq) else None,
+                                  gamma_k=[dev(g) for g in gk] if any(g is not None for g in gk) else None,
+                                  rot_q=dev(rot_q), rot_k=dev(rot_k), static_scratch=static)
+        mx, rr = oracle.err_stats(got.cpu().numpy(), want)
+        assert mx <= 2e-2 and rr <= 1e-3, (i, mx, rr)
+
+
+def test_dense_large_palettes_tall_tile_random(dthip, oracle, torch_cuda):
+    """128- and 256-entry palettes with small blocks on problems large enough for the 256-token x 128-feature tile
+    (per-row palette tables, weight staging by one wave per SIMD): random ragged shapes against the oracle."""
+    torch = torch_cuda
+    rng = np.random.default_rng(107)
+    for i in range(12):
+        q = int(rng.choice([7, 8]))
+        nib = int(rng.choice([64, 512, 1024, 4096]))
+        K = int(rng.choice([128, 256, 512, 768]))
+        M = int(rng.integers(2300, 3100))
+        N = int(rng.integers(2200, 2600))
+        print("dense tall tile", i, q, nib, M, K, N, flush=True)
+        packed, _, _ = oracle.synth_qx_weight(rng, N, K, q, nib, 0.05)
+        w = dthip.QxTensor.from_packed(packed, q, nib, (N, K))
+        x = f16(rng.standard_normal((M, K)))
+        b = f16(rng.standard_normal(N) * 0.05) if rng.random() < 0.7 else None
+        got = dthip.dense_multi(to_dev(torch, x), [w], [None if b is None else to_dev(torch, b)])[0].cpu().numpy()
+        mx, rr = oracle.err_stats(got, oracle.C.dense_qx(x, packed, q, nib, N, b))
+        assert mx <= 2e-2 and rr <= 1e-3, (i, mx, rr)
