@@ -551,7 +551,7 @@ def main():
         return e0.elapsed_time(e1) / iters
 
     # the standalone norm / RoPE pass works in place: it gets a copy of Q and K of its own, never the step's buffer
-    qkv_prep = qkv.clone()
+    qkv_prep = qkv.float().half()  # (elementwise kernels, not a device copy: --copy-calibration counts those)
     qp4, kp4 = qkv_prep[:, 0].unsqueeze(0), qkv_prep[:, 1].unsqueeze(0)
 
     def k_prep():
