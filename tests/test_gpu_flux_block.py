@@ -319,3 +319,80 @@ def test_flux_step_full_size_sampled(dthip, oracle):
     mx, rr = oracle.err_stats(got_out[rows], want_out)
     print("out max-abs", mx, "rel-rms", rr, flush=True)
     assert mx <= 2e-2 and rr <= 2e-3, (mx, rr)
+
+
+def test_four_host_threads_on_four_streams(dthip, oracle):
+    """The reference runs a model on up to four concurrent streams (maxConcurrency = .limit(4),
+    Models/UNetProtocol.swift:2011).  Four host threads, each with a stream and inputs of its own, run the same
+    chain -- palettized QKV projection with the fused head epilogue, attention (one thread's launch small enough to
+    be key-split, each call with a workspace of its own), output projection -- several times over at once; every
+    thread's result must equal, bit for bit, what the same chain gives when it runs alone."""
+    import threading
+
+    import torch
+
+    H, D, q, nib = 4, 128, 6, 4096
+    C = H * D
+    rng = np.random.default_rng(2011)
+    f16 = lambda a: np.asarray(a, dtype=np.float16)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    ws = {}
+    for name in ("q", "k", "v", "o"):
+        packed, _, _ = oracle.synth_qx_weight(rng, C, C, q, nib)
+        ws[name] = dthip.QxTensor.from_packed(packed, q, nib, (C, C))
+    gam = dev(f16(1 + 0.02 * rng.standard_normal(D)))
+    sizes = [1300, 900, 4096, 700]  # (4 heads x 4096 tokens is split along the keys by the library's own estimate)
+    assert dthip.lib().dt_sdpa_workspace_bytes(1, H, H, D, 4096, 4096, 0, 0) > 0
+    rots = [dev(f16(dthip.WanRotaryPositionEmbedding(1, S, 1, channels=D))) for S in sizes]
+    xs = [dev(f16(rng.standard_normal((S, C)))) for S in sizes]
+
+    def chain(i, stream):
+        S = sizes[i]
+        epi = [dthip.HeadEpilogue(gam, rots[i], 0, 1e-6, D), dthip.HeadEpilogue(gam, rots[i], 0, 1e-6, D), None]
+        qo, ko, vo = dthip.dense_multi(xs[i], [ws["q"], ws["k"], ws["v"]], [None] * 3, epilogues=epi, stream=stream)
+        att = dthip.sdpa_segments([qo.view(1, S, H, D)], [ko.view(1, S, H, D)], [vo.view(1, S, H, D)], 1 / np.sqrt(D),
+                                  stream=stream)
+        return dthip.dense_multi(att.view(S, C), [ws["o"]], [None], stream=stream)[0]
+
+    torch.cuda.synchronize()
+    alone = []
+    for i in range(4):
+        alone.append(chain(i, None))
+        torch.cuda.synchronize()
+    results, errors = [None] * 4, []
+
+    def worker(i):
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            out = None
+            for _ in range(6):
+                out = chain(i, stream)
+            stream.synchronize()
+            results[i] = out
+        except Exception as e:  # surfaces in the main thread below
+            errors.append((i, repr(e)))
+
+    print("four threads, four streams", flush=True)
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for i in range(4):
+        assert torch.equal(results[i], alone[i]), i
+    # and the chain itself is right: one thread's result against the oracle
+    i, S = 1, sizes[1]
+    x = xs[i].cpu().numpy()
+    heads = lambda a: a.reshape(S, H, D)
+    pk = {n: oracle.C.depalettize(q, nib, C * C, ws[n].data.cpu().numpy()[: dthip.qx_bytes(q, nib, C * C)]).reshape(C, C) for n in ws}
+    g, r = gam.cpu().numpy(), rots[i].cpu().numpy()
+    rq = oracle.C.cmul(oracle.C.rmsnorm(heads(oracle.C.dense(x, pk["q"], None)), g, 1e-6), r)
+    rk = oracle.C.cmul(oracle.C.rmsnorm(heads(oracle.C.dense(x, pk["k"], None)), g, 1e-6), r)
+    rv = heads(oracle.C.dense(x, pk["v"], None))
+    att = oracle.C.sdpa(rq[None], rk[None], rv[None], 1 / np.sqrt(D)).reshape(S, C)
+    want = oracle.C.dense(att, pk["o"], None)
+    mx, rr = oracle.err_stats(results[i].cpu().numpy(), want)
+    assert mx <= 2e-2 and rr <= 2e-3, (mx, rr)
