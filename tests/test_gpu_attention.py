@@ -775,3 +775,40 @@ def test_sdpa_quantized_level_flags_are_permissions(dthip, oracle, torch_cuda):
     assert torch.equal(f16_only, quantized)
     mx, rr = oracle.err_stats(quantized.cpu().numpy(), oracle.C.sdpa(q, k, v, scale))
     assert mx <= MAX_ABS and rr <= REL_RMS, (mx, rr)
+
+
+def test_sdpa_key_split_replays_as_hip_graph(dthip, oracle, torch_cuda, monkeypatch):
+    """A key-split attention launch (counter reset by a fill kernel, partial results through the workspace, fold by
+    the last piece to arrive) captured in a HIP graph with fused query / key prep: every replay, with eager calls
+    and synchronisations in between and the outputs cleared each time, gives the eager result bit for bit."""
+    torch = torch_cuda
+    monkeypatch.setenv("DT_SDPA_KEY_SPLIT", "always")
+    rng = np.random.default_rng(911)
+    B, S, H, D = 1, 1500, 3, 128
+    q, k, v = rand_qkv(rng, B, S, S, H, H, D)
+    g = to_dev(torch, f16(1 + 0.05 * rng.standard_normal(D)))
+    rot = to_dev(torch, f16(dthip.WanRotaryPositionEmbedding(1, S, 1, channels=D)))
+    qd, kd, vd = (to_dev(torch, t) for t in (q, k, v))
+    out = torch.zeros((B, S, H, D), dtype=torch.float16, device="cuda")
+    call = lambda: dthip.sdpa_segments([qd], [kd], [vd], 1 / np.sqrt(D), gamma_q=[g], gamma_k=[g], rot_q=rot, rot_k=rot,
+                                       out=out)
+    print("key-split attention as hip graph", flush=True)
+    call()
+    torch.cuda.synchronize()
+    want = out.clone()
+    assert float(want.abs().max()) > 0
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for _ in range(4):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+        call()  # eager work between the replays
+        torch.cuda.synchronize()
