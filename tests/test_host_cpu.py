@@ -103,3 +103,48 @@ def test_operator_surface_argument_checks(dthip):
     d = dthip.Dense(count=8, noBias=True, name="x_q")
     with pytest.raises(RuntimeError, match="weight not loaded"):
         d(None)
+
+
+def test_header_is_plain_c_and_links(dthip, tmp_path):
+    """include/dt_hip.h is what a C (or Swift, through the module map) caller sees: it must compile as C99 on its
+    own, and a C program linked against libdthip.so must be able to call the host-only entry points."""
+    import shutil
+    import subprocess
+
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include "dt_hip.h"
+#include <stdio.h>
+#include <string.h>
+int main(void) {
+  dt_qx_weight w; dt_view4 v; dt_seq_segment s; dt_head_epilogue e; dt_dense_post p; dt_dense_group g;
+  memset(&w, 0, sizeof w); memset(&v, 0, sizeof v); memset(&s, 0, sizeof s); memset(&e, 0, sizeof e);
+  memset(&p, 0, sizeof p); memset(&g, 0, sizeof g);
+  (void)w; (void)v; (void)s; (void)e; (void)p; (void)g;
+  /* every entry point is declared with C linkage and takes only plain pointers and sizes */
+  typedef void (*fn_t)(void);
+  fn_t fns[] = {FNS};
+  if (sizeof fns / sizeof fns[0] != NFNS) return 2;
+  if (DT_OK != 0 || DT_INVALID != -1 || DT_NO_KERNEL != -2 || DT_OOM != -3) return 3;  /* ccv's exec status values */
+  printf("%s %lld %zu\n", dt_version(), (long long)dt_qx_bytes(6, 4096, 3072LL * 3072),
+         dt_sdpa_workspace_bytes(1, 24, 24, 128, 4608, 4608, 1, 0));
+  return 0;
+}
+''')
+    inc = os.path.join(ROOT, "include")
+    text = src.read_text().replace("FNS", ", ".join(f"(fn_t){name}" for name in dthip.ABI_SYMBOLS), 1)
+    src.write_text(text.replace("NFNS", str(len(dthip.ABI_SYMBOLS))))
+    subprocess.check_call([cc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-fsyntax-only", "-I", inc, str(src)])
+    libdir = os.path.dirname(dthip.LIB_PATH)
+    exe = tmp_path / "abi"
+    subprocess.check_call([cc, "-std=c99", "-I", inc, str(src), "-o", str(exe), "-L", libdir, "-ldthip",
+                           "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"])
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stderr
+    ver, qx, ws = out.stdout.split()[-3:] if len(out.stdout.split()) >= 3 else (None, None, None)
+    assert "gfx950" in out.stdout
+    assert int(qx) == dthip.qx_bytes(6, 4096, 3072 * 3072)
+    assert int(ws) == 4608 * 24 * 128 * 2
