@@ -31,3 +31,4 @@ def test_store_to_dense(tmp_path, dthip, oracle):
     got = layer(torch.from_numpy(X).cuda()).cpu().numpy()
     mx, rr = oracle.err_stats(got, oracle.C.dense_qx(X, packed, q, nib, N, bias))
     assert mx <= 2e-2 and rr <= 1e-3
+

@@ -148,3 +148,19 @@ int main(void) {
     assert "gfx950" in out.stdout
     assert int(qx) == dthip.qx_bytes(6, 4096, 3072 * 3072)
     assert int(ws) == 4608 * 24 * 128 * 2
+
+
+def test_cpp_operator_mirror_compiles(dthip, tmp_path):
+    """include/dt_hip.hpp (the C++ operator objects above the C ABI) compiles on its own as C++17 with warnings as
+    errors, and the check program built from it exists beside the library after a build."""
+    import shutil
+    import subprocess
+
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        pytest.skip("no C++ compiler")
+    src = tmp_path / "mirror.cpp"
+    src.write_text('#include "dt_hip.hpp"\nint main() { dt::Dense d(8, true); return d.count == 8 ? 0 : 1; }\n')
+    subprocess.check_call([cxx, "-std=c++17", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I",
+                           os.path.join(ROOT, "include"), str(src)])
+    assert os.path.exists(os.path.join(os.path.dirname(dthip.LIB_PATH), "dt_cpp_check"))
