@@ -802,6 +802,7 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
   issue_idx(WS[1]);  // tile 3
   __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
   __syncthreads();
+  if constexpr (MODE == kPlainF16) issue_pair(XsB, WpB, 1);  // (the loop issues pair q + 2 from the middle of pair q)
 #pragma unroll
   for (int i = 0; i < TN; i++) read_w(0, i, WpA, 0, 0, 0);
 #pragma unroll
@@ -884,6 +885,44 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
         st(k - NF);
       }
     };
+    if constexpr (!packed) {
+      // Plain fp16 weights: both operands arrive by transfer and nothing is written to LDS by the waves, so one
+      // barrier per pair of K-tiles is enough, and it sits in the middle of the odd iteration: by then the pair in
+      // flight has had two iterations to land, the reads of this pair's last k-step were issued half an
+      // iteration ago, and what follows the barrier is exactly what needs it -- the first reads from the other
+      // slot and the transfer of the pair after next into this one.
+      constexpr int RPS = (NF + NM - 1) / NM;            // fragment reads per MFMA, front-loaded
+      constexpr int PPS = (AP + BP + NM - 1) / NM;       // transfer parts per MFMA
+#pragma unroll
+      for (int m = 0; m < NM; m++) {
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(0, m / TM, m % TM);
+#pragma unroll
+        for (int r = m * RPS; r < (m + 1) * RPS; r++)
+          if (r < NF) read0(r);
+      }
+      if (par) {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+        __syncthreads();
+      }
+#pragma unroll
+      for (int m = 0; m < NM; m++) {
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(1, m / TM, m % TM);
+#pragma unroll
+        for (int r = m * RPS; r < (m + 1) * RPS; r++)
+          if (r < NF) read1(r);
+        if (par) {
+          // this iteration's slot is free from the barrier on: the pair after next goes into it
+#pragma unroll
+          for (int q = m * PPS; q < (m + 1) * PPS; q++)
+            if (q < AP + BP) issue_pair_part(xs, wp, (t >> 1) + 2, q);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      return;
+    }
     const int n0 = NF + (ns0 > 2 * NF ? ns0 : 2 * NF);
     const int n1 = NF + (ns1 > 2 * NF ? ns1 : 2 * NF);
 #pragma unroll
@@ -924,6 +963,11 @@ __global__ void __launch_bounds__(512) dense_qx_kernel(const DenseArgs a) {
     iteration(t + 1, 1, XsA, WpA, XsB, WpB);
   }
 
+  if constexpr (MODE == kPlainF16) {
+    // the loop's last barrier lies before the last reads (and every transfer was waited for ahead of it)
+    __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+    __syncthreads();
+  }
   dense_epilogue<WN, WM, POST>(acc, smem, wave, lane, n0 + wn * WN, (int64_t)m0 + wm * WM, w, g.m);
 }
 
