@@ -9,7 +9,8 @@
 // activation / gate / fp32 residual).
 //
 // Tile: BM x BN outputs per 512-thread workgroup (8 waves, two per SIMD, each
-// a BN/2 x BM/4 slice), K-tiles of 32 processed in pairs; one barrier per K-tile.
+// a BN/2 x BM/4 slice), K-tiles of 32 processed in pairs; one barrier per K-tile
+// (per pair with plain fp16 weights, which no wave writes to LDS itself).
 #include "dt_dense_launch.h"
 
 namespace dt {

@@ -308,7 +308,7 @@ DT_EXPORT dt_status dt_sdpa_f16_static(dt_stream stream, int32_t B, int32_t Hq, 
   if (sh.need > (size_t)DT_SDPA_STATIC_SCRATCH_BYTES) return DT_OOM;  // beyond the fixed array: use dt_sdpa_f16
   if (const dt_status ready = device_ready(); ready != DT_OK) return ready;
   // the staging bytes are a must; the key-split form's room is used if the array still has it
-  size_t give = dt_sdpa_workspace_bytes(B, Hq, Hk, D, sh.Sq, sh.Skv, sh.prep ? 1 : 0, Wo ? 1 : 0);
+  size_t give = dt_sdpa_workspace_bytes(B, Hq, Hk, D, sh.Sq, sh.Skv, sh.kprep ? 1 : 0, Wo ? 1 : 0);
   if (give > (size_t)DT_SDPA_STATIC_SCRATCH_BYTES) give = sh.need;
   void* ws = nullptr;
   if (give > 0) {
