@@ -28,7 +28,7 @@ PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
 # counters read for a 256 MiB device copy (x2.00 and x1.00); the summary is profiles/bench_flux_block_counters.txt
-MEASURED_TRAFFIC_BYTES = {"dense_qkv": 3.742e8, "sdpa": 1.326e8}
+MEASURED_TRAFFIC_BYTES = {"dense_qkv": 3.742e8, "sdpa": 1.327e8}
 TRAFFIC_SOURCE = "profiles/bench_flux_block_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script; not measured by this run)"
 SDPA_NAME = "sdpa_kernel<128> S=4608 H=24"
 QKV_NAME = "dense_qx_kernel<6,256,256> M=4096+512 N=3x3072 K=3072 (fused norm/RoPE epilogue)"
