@@ -232,6 +232,41 @@ def test_dense_flux_qkv_full_size_sampled(dthip, oracle, torch_cuda):
         assert float((a.float() * 2 - b.float()).abs().max()) <= 2.0 ** -23
 
 
+def test_dense_plain_fp16_full_size_equals_palettized(dthip, oracle, torch_cuda):
+    """Plain fp16 weights at the benchmark's shape (M 4608, K 3072, three N 3072 weights in one launch, the plain
+    path's own schedule: one barrier per pair of K-tiles): sampled rows against the oracle, and bit for bit what the
+    palettized path gives for the same effective weights (both accumulate the k-steps in the same order)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(41)
+    M, K, N, q, nib = 4608, 3072, 3072, 6, 4096
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    ws, biases = [], []
+    for i in range(3):
+        w, _ = make_weight(dthip, oracle, rng, N, K, q, nib)
+        ws.append(w)
+        biases.append((rng.standard_normal(N) * 0.02).astype(np.float16))
+    plain = [dthip.QxTensor.from_f16(w.dequantize()) for w in ws]
+    xd = to_dev(torch, X)
+    bd = [to_dev(torch, b) for b in biases]
+    print("dense plain fp16 full size", flush=True)
+    got = dthip.dense_multi(xd, plain, bd)
+    ref = dthip.dense_multi(xd, ws, bd)
+    rows = np.sort(rng.choice(M, size=16, replace=False))
+    rows[0], rows[-1] = 0, M - 1
+    for i in range(3):
+        assert torch.equal(got[i], ref[i]), i
+        W = plain[i].data.cpu().numpy()
+        want = oracle.C.dense(np.ascontiguousarray(X[rows]), W, biases[i])
+        mx, rr = oracle.err_stats(got[i].cpu().numpy()[rows], want)
+        assert mx <= MAX_ABS and rr <= REL_RMS, (i, mx, rr)
+    # a launch of less than two pairs of K-tiles, and one whose token count leaves a ragged last tile
+    for (m, k) in ((300, 64), (1500, 128), (4100, 192)):
+        x = to_dev(torch, rng.standard_normal((m, k)).astype(np.float16))
+        w, _ = make_weight(dthip, oracle, rng, 512, k, q, 512)
+        p = dthip.QxTensor.from_f16(w.dequantize())
+        assert torch.equal(dthip.dense_multi(x, [p], [None])[0], dthip.dense_multi(x, [w], [None])[0]), (m, k)
+
+
 @pytest.mark.parametrize("M,head_dim,q,nib", [(700, 128, 6, 4096), (300, 128, 8, 16384), (130, 64, 6, 4096),
                                               (1024, 128, 6, 4096), (4200, 128, 5, 1024)])
 def test_dense_fused_head_norm_rope(dthip, oracle, torch_cuda, M, head_dim, q, nib):
